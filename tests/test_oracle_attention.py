@@ -1,0 +1,125 @@
+"""Pins oracle/attention.py: dense special case, token-mask equivalence, PV-skip rule, end-to-end API."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import api, attention as at, maskpred as mp, vquant as vq
+from oracle import rounding as R
+
+
+def _inputs(seed, b, h, n, d, tag):
+    rng = np.random.default_rng(seed)
+    mk = lambda s: R.round_to(rng.standard_normal((b, h, n, d)) * s, tag)
+    return mk(1.0), mk(1.0) + 0.5, mk(1.0)
+
+
+def _dequantised(res, n, d):
+    """Float tensors the kernel effectively multiplies: q8*q_scale, k8*k_scale, v8*v_scale."""
+    q = res["q8"].astype(np.float64) * np.repeat(res["q_scale"].astype(np.float64), 128, axis=2)[:, :, :n, None]
+    k = res["k8"].astype(np.float64) * np.repeat(res["k_scale"].astype(np.float64), 64, axis=2)[:, :, :n, None]
+    v = vq.dequant(res["v8"])[:, :, :n].astype(np.float64) * res["v_scale"].astype(np.float64)[:, :, None, :]
+    return torch.from_numpy(q), torch.from_numpy(k), torch.from_numpy(v)
+
+
+def _token_mask(block_map, n):
+    """Token-level mask of a 128x64 block map (what block_map_to_mask builds, utils.py:424-432)."""
+    m = np.repeat(np.repeat(block_map, 128, axis=2), 64, axis=3)
+    return torch.from_numpy(m[:, :, :n, :n])
+
+
+@pytest.mark.parametrize("tag,d,n", [(R.BF16, 128, 384), (R.FP16, 64, 300)])
+def test_all_blocks_reduces_to_dense_sdpa(tag, d, n):
+    q, k, v = _inputs(0, 1, 2, n, d, tag)
+    res = api.spas_sage2_attn_meansim_topk(q, k, v, tag, topk=1.0)
+    assert res["map"].all() and np.array_equal(res["pv_count"], res["valid"])
+    qd, kd, vd = _dequantised(res, n, d)
+    ref = torch.nn.functional.scaled_dot_product_attention(qd, kd, vd).numpy()
+    met = at.precision_metric(res["out"], ref)
+    # remaining error: e4m3 rounding of P (numerator only) and the output rounding
+    assert met["Cossim"] > 0.9995 and met["L1"] < 0.03, met
+    # and against the un-quantised inputs (reported accuracy of the method itself)
+    ref2 = torch.nn.functional.scaled_dot_product_attention(
+        torch.from_numpy(q).double(), torch.from_numpy(k).double(), torch.from_numpy(v).double()).numpy()
+    assert at.precision_metric(res["out"], ref2)["Cossim"] > 0.999
+
+
+def test_block_map_equals_token_masked_sdpa():
+    tag, d, n = R.BF16, 64, 512
+    q, k, v = _inputs(1, 1, 2, n, d, tag)
+    rng = np.random.default_rng(2)
+    mask = rng.random((1, 2, 4, 8)) < 0.4
+    mask[:, :, np.arange(4), 2 * np.arange(4)] = True
+    res = api.block_sparse_sage2_attn(q, k, v, mask.astype(np.int32), tag)
+    qd, kd, vd = _dequantised(res, n, d)
+    ref = torch.nn.functional.scaled_dot_product_attention(qd, kd, vd, attn_mask=_token_mask(mask, n)).numpy()
+    met = at.precision_metric(res["out"], ref)
+    assert met["Cossim"] > 0.9995 and met["L1"] < 0.03, met
+    assert res["written"].all()
+
+
+def test_kernel_causal_flag_equals_token_causal_sdpa():
+    tag, d, n = R.FP16, 64, 512
+    q, k, v = _inputs(3, 1, 1, n, d, tag)
+    res = api.spas_sage2_attn_meansim_topk(q, k, v, tag, topk=1.0, is_causal=True, kernel_causal=True)
+    qd, kd, vd = _dequantised(res, n, d)
+    ref = torch.nn.functional.scaled_dot_product_attention(qd, kd, vd, is_causal=True).numpy()
+    assert at.precision_metric(res["out"], ref)["Cossim"] > 0.9995
+    # reference behaviour (kernel flag False): causality only at block granularity
+    res_b = api.spas_sage2_attn_meansim_topk(q, k, v, tag, topk=1.0, is_causal=True, kernel_causal=False)
+    cm = mp.causal_block_mask(4, 8)
+    ref_b = torch.nn.functional.scaled_dot_product_attention(
+        qd, kd, vd, attn_mask=_token_mask(np.broadcast_to(cm, (1, 1, 4, 8)), n)).numpy()
+    assert at.precision_metric(res_b["out"], ref_b)["Cossim"] > 0.9995
+
+
+def test_partial_blocks_and_empty_rows():
+    tag, d, n = R.BF16, 64, 333            # partial last Q block (77 rows) and K block (13 rows)
+    q, k, v = _inputs(4, 1, 1, n, d, tag)
+    mask = np.ones((1, 1, 3, 6), np.int32)
+    mask[0, 0, 1] = 0                       # a row block with no selected K block stays unwritten
+    res = api.block_sparse_sage2_attn(q, k, v, mask, tag)
+    assert list(res["written"][0, 0]) == [True, False, True]
+    assert np.all(res["out"][0, 0, 128:256] == 0)
+    qd, kd, vd = _dequantised(res, n, d)
+    ref = torch.nn.functional.scaled_dot_product_attention(qd, kd, vd).numpy()
+    sel = np.r_[0:128, 256:n]
+    assert at.precision_metric(res["out"][0, 0, sel], ref[0, 0, sel])["Cossim"] > 0.9995
+
+
+def test_pv_threshold_skip_rule():
+    """Two-scale example: K blocks 0..1 carry large scores, blocks 2..3 tiny ones, 4..5 close the row.
+
+    With the running maximum set by block 0, every later middle block has m_blk far below m.
+    Threshold t skips a middle block iff max_rows(m_blk - m_prev) + t <= 0 (sm89.cuh:353)."""
+    tag, d, n = R.FP16, 64, 384
+    rng = np.random.default_rng(5)
+    q = R.round_to(np.abs(rng.standard_normal((1, 1, n, d))) + 0.5, tag)
+    k = R.round_to(rng.standard_normal((1, 1, n, d)) * 0.05, tag)
+    k[0, 0, :64] += 6.0                                  # block 0 dominates every row
+    v = R.round_to(rng.standard_normal((1, 1, n, d)), tag)
+    mask = np.ones((1, 1, 3, 6), np.int32)
+    hi = api.block_sparse_sage2_attn(q, k, v, mask, tag, pvthreshd=1e6)
+    lo = api.block_sparse_sage2_attn(q, k, v, mask, tag, pvthreshd=5.0)
+    # 6 blocks per row: 4 middle (skippable) + 2 final (never skipped); block 0 always raises the max
+    assert np.all(hi["pv_count"] == 6)
+    assert np.all(lo["pv_count"] == 3), lo["pv_count"]
+    # skipped blocks carried < 2^-5 of the weight... the result changes only slightly
+    assert at.precision_metric(lo["out"], hi["out"])["Cossim"] > 0.99
+    # the first block raises m from the -5e6 sentinel, i.e. delta ~ 5e6: it survives t = -1e6 but not t = -1e7
+    assert np.all(api.block_sparse_sage2_attn(q, k, v, mask, tag, pvthreshd=-1e6)["pv_count"] == 3)
+    assert np.all(api.block_sparse_sage2_attn(q, k, v, mask, tag, pvthreshd=-1e7)["pv_count"] == 2)
+
+
+def test_topk_api_end_to_end_small():
+    tag, d, n = R.BF16, 64, 1024
+    q, k, v = _inputs(6, 1, 2, n, d, tag)
+    res = api.spas_sage2_attn_meansim_topk(q, k, v, tag, topk=0.5)
+    assert res["lut"].shape == (1, 2, 8, 16) and np.all(res["valid"] == 8)
+    assert abs(res["sparsity"] - 0.5) < 1e-12
+    qd, kd, vd = _dequantised(res, n, d)
+    ref = torch.nn.functional.scaled_dot_product_attention(qd, kd, vd, attn_mask=_token_mask(res["map"], n)).numpy()
+    assert at.precision_metric(res["out"], ref)["Cossim"] > 0.9995
+    res_c = api.spas_sage2_attn_meansim_topk(q, k, v, tag, topk=0.5, is_causal=True)
+    assert list(res_c["valid"][0, 0]) == [2, 4, 6, 8, 8, 8, 8, 8]
+    tot = float(res_c["valid"].sum())
+    assert abs(res_c["sparsity"] - (1 - tot / (9 * 8 * 2))) < 1e-12      # causal denominator (nk+2)//2
