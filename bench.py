@@ -1,0 +1,201 @@
+#!/usr/bin/env python3
+"""Headline benchmark: spas_sage2_attn_meansim_topk_cuda on one MI355X.
+
+One step = one call of the operator (K mean, mask prediction + INT8 quantisation, V FP8 quantisation,
+block-sparse attention) on the headline configuration cfg4 (B=1, H=32, N=32768, D=128, bf16, causal,
+topk=0.5, pvthreshd=50) with synthetic inputs already resident in HBM.
+
+Prints ONE JSON line.  value = dense-equivalent TOPS of the whole step (4*B*H*N^2*D/2 per step time).
+Extra keys: the attention kernel alone, the mask-prediction/quantisation stages (us and GB/s), the dense FP16
+comparator built in the same library, the MFMA roofline of the attention kernel and a CPU baseline (the numpy
+oracle on a bounded sample).
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+import torch
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+PEAK_MFMA_8BIT = 5.0e15   # MI355X dense INT8 = FP8 MFMA peak, op/s
+PEAK_HBM = 8.0e12
+
+
+def parse():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=10)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--config", default="cfg4", help="workload (cfg1..cfg5); the headline is cfg4")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-dense", action="store_true")
+    ap.add_argument("--attn-only", action="store_true",
+                    help="time only the attention kernel launches (for rocprofv3 runs of the dominant kernel)")
+    return ap.parse_args()
+
+
+def cpu_baseline(cfg):
+    """numpy oracle on a bounded sample of the headline workload: one head, N = 4096."""
+    import numpy as np
+    from oracle import api as oapi
+    from spargeattn_amd import workloads as W
+    n = 4096
+    q, k, v = W.make_qkv(cfg, device="cpu", shrink=dict(B=1, H=1, N=n))
+    qn, kn, vn = (t.float().numpy() for t in (q, k, v))
+    tag = "bf16" if cfg.dtype == torch.bfloat16 else "fp16"
+    threads = os.cpu_count() or 1
+    t0 = time.perf_counter()
+    oapi.spas_sage2_attn_meansim_topk(qn, kn, vn, tag, is_causal=cfg.is_causal, topk=cfg.topk, pvthreshd=cfg.pvthreshd)
+    dt = time.perf_counter() - t0
+    flop = 4.0 * n * n * cfg.D * (0.5 if cfg.is_causal else 1.0)
+    return {"value": flop / dt / 1e12, "unit": "dense-equiv TOPS", "cores": threads, "kind": "port",
+            "sample": f"numpy oracle (BLAS threads = host cores), full operator on B=1,H=1,N={n},D={cfg.D} of the "
+                      f"{cfg.name} generator, {dt:.1f} s"}
+
+
+def main():
+    args = parse()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)", file=sys.stderr)
+        sys.exit(2)
+    import spargeattn_amd as sa
+    from spargeattn_amd import core, _lib, workloads as W
+
+    cfg = W.CONFIGS[args.config]
+    if cfg.api != "topk":
+        print("bench.py times the top-k operator; pick cfg1, cfg3, cfg4 or cfg5", file=sys.stderr)
+        sys.exit(2)
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    _lib.load()
+    q, k, v = W.make_qkv(cfg, device=dev)
+    B, H, N, D = q.shape
+    nq, nk = (N + 127) // 128, (N + 63) // 64
+    dense_flop = 4.0 * B * H * N * N * D * (0.5 if cfg.is_causal else 1.0)
+
+    def step():
+        return sa.spas_sage2_attn_meansim_topk_cuda(q, k, v, is_causal=cfg.is_causal, topk=cfg.topk,
+                                                    pvthreshd=cfg.pvthreshd)
+
+    # ---- stage events (recorded on the stream the kernels are launched on) -------------------------------
+    names = ["km", "maskpred", "vquant", "attn", "end"]
+    marks = []
+
+    def hook(name):
+        e = torch.cuda.Event(enable_timing=True)
+        e.record()
+        marks.append((name, e))
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+
+    if args.attn_only:
+        # the dominant kernel alone, on the tensors the operator would hand it
+        km = _lib.km_mean(k)
+        from spargeattn_amd import utils
+        lut, valid, q8, qs, k8, ks = utils.get_block_map_meansim_fuse_quant(
+            q, k, km, is_causal=cfg.is_causal, simthreshd1=-0.1, cdfthreshd=None, topk=cfg.topk, return_lut=True)
+        v8, vs = _lib.v_quant_fp8(v.to(torch.float16))
+        o = torch.empty_like(q)
+        pvt = torch.full((H,), float(cfg.pvthreshd), device=dev)
+        run = lambda: _lib.block_sparse_attn(q8, k8, v8, o, lut, valid, pvt, qs, ks, vs, 1.0 / D ** 0.5)
+        for _ in range(args.warmup):
+            run()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            run()
+        torch.cuda.synchronize()
+        dt = (time.perf_counter() - t0) / args.steps
+        print(json.dumps({"attn_only_ms": dt * 1e3, "dense_equiv_tops": dense_flop / dt / 1e12}))
+        return
+
+    core._stage_hook = hook
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+    core._stage_hook = None
+    step_s = (t1 - t0) / args.steps
+
+    stage_ms = {n: 0.0 for n in names[:-1]}
+    for i in range(0, len(marks), len(names)):
+        grp = marks[i:i + len(names)]
+        for (n0, e0), (_, e1) in zip(grp[:-1], grp[1:]):
+            stage_ms[n0] += e0.elapsed_time(e1)
+    for n0 in stage_ms:
+        stage_ms[n0] /= args.steps
+    attn_s = stage_ms["attn"] * 1e-3
+
+    # ---- executed work of the attention kernel ----------------------------------------------------------------
+    from spargeattn_amd import utils
+    km = _lib.km_mean(k)
+    lut, valid, *_ = utils.get_block_map_meansim_fuse_quant(q, k, km, is_causal=cfg.is_causal, simthreshd1=-0.1,
+                                                            cdfthreshd=None, topk=cfg.topk, return_lut=True)
+    sel_blocks = int(valid.sum().item())
+    executed_ops = sel_blocks * 2.0 * (128 * 64 * D) * 2.0
+    del lut, valid, km
+
+    # ---- algorithmic bytes of mask prediction + quantisation (read Q once, K twice, V twice; write Q8,K8,V8) ---
+    elt = B * H * N * D
+    mp_bytes = 2 * elt * (1 + 2) + 2 * elt + (nq + nk) * B * H * D * 2 + 4 * B * H * nq * nk
+    vq_bytes = 2 * elt * 2 + elt
+    mp_ms = stage_ms["km"] + stage_ms["maskpred"]
+
+    out = {
+        "metric": "dense-equiv TOPS + MFMA util % at N=32K,D=128 causal topk=0.5; mask-pred us",
+        "value": dense_flop / step_s / 1e12,
+        "unit": "dense-equiv TOPS (4*B*H*N^2*D/2 per step time)",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": step_s * 1e3,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "int8 QK^T + fp8-e4m3 PV (fp32 softmax/accumulate), bf16 in/out",
+        "data": "synthetic (seeded generator, see spargeattn_amd/workloads.py)",
+        "config": {"workload": f"{cfg.name}: spas_sage2_attn_meansim_topk_cuda B={B} H={H} N={N} D={D} "
+                               f"{'causal' if cfg.is_causal else 'non-causal'} topk={cfg.topk} pvthreshd={cfg.pvthreshd}",
+                   "selected_blocks": sel_blocks, "block_density": sel_blocks / (B * H * nq * nk)},
+        "attn_kernel": {"ms": stage_ms["attn"], "dense_equiv_tops": dense_flop / attn_s / 1e12,
+                        "executed_tops": executed_ops / attn_s / 1e12,
+                        "mfma_util_pct": 100.0 * executed_ops / attn_s / PEAK_MFMA_8BIT},
+        "mask_pred": {"us": mp_ms * 1e3, "km_us": stage_ms["km"] * 1e3, "pool_quant_select_us": stage_ms["maskpred"] * 1e3,
+                      "algorithmic_GB": mp_bytes / 1e9, "GBps": mp_bytes / (mp_ms * 1e-3) / 1e9,
+                      "hbm_frac": mp_bytes / (mp_ms * 1e-3) / PEAK_HBM},
+        "v_quant": {"us": stage_ms["vquant"] * 1e3, "GBps": vq_bytes / (stage_ms["vquant"] * 1e-3) / 1e9},
+        "roofline": {"kernel": "block_sparse_attn_kernel<128,bf16>", "bound": "mfma",
+                     "achieved": executed_ops / attn_s / 1e12, "peak": PEAK_MFMA_8BIT / 1e12, "unit": "TFLOP/s",
+                     "frac": executed_ops / attn_s / PEAK_MFMA_8BIT, "traffic": None,
+                     "note": "achieved = executed INT8+FP8 MFMA ops (selected blocks * 2*128*64*D*2) / HIP-event time of "
+                             "the kernel inside the timed steps; peak = MI355X dense 8-bit MFMA"},
+    }
+
+    if not args.no_dense:
+        qh, kh, vh = q.to(torch.float16), k.to(torch.float16), v.to(torch.float16)
+        vt = _lib.v_tiles_f16(vh)
+        oh = torch.empty_like(qh)
+        sc = 1.0 / D ** 0.5
+        for _ in range(max(1, args.warmup)):
+            _lib.dense_attn_f16(qh, kh, vt, sc, is_causal=cfg.is_causal, out=oh)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            _lib.dense_attn_f16(qh, kh, vt, sc, is_causal=cfg.is_causal, out=oh)
+        torch.cuda.synchronize()
+        dn = (time.perf_counter() - t0) / args.steps
+        out["dense_fp16"] = {"ms": dn * 1e3, "tops": dense_flop / dn / 1e12,
+                             "speedup_step": dn / step_s, "speedup_attn_kernel": dn / attn_s}
+        del qh, kh, vh, vt, oh
+
+    if not args.no_cpu_baseline:
+        out["cpu_baseline"] = cpu_baseline(cfg)
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

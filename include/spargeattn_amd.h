@@ -1,0 +1,109 @@
+/*
+ * spargeattn_amd.h - C ABI of the MI355X (gfx950) SpargeAttn hot path.
+ *
+ * One function per stage of
+ *   spas_sage2_attn_meansim_topk_cuda   (spas_sage_attn/core.py:105-169)
+ *   block_sparse_sage2_attn_cuda        (spas_sage_attn/core.py:171-233)
+ * of thu-ml/SpargeAttn.  Every function takes raw DEVICE pointers, explicit
+ * sizes, enum ints and a HIP stream (hipStream_t passed as void*); it launches
+ * asynchronously on that stream, allocates nothing, synchronises nothing and
+ * keeps no state.  Tensors are contiguous in the "HND" layout (B,H,N,D).
+ * Return value: SPG_OK or an error code; spg_last_error() gives the message of
+ * the last failure on the calling thread.
+ *
+ * Block geometry (fixed, as on the reference's non-Hopper path, core.py:128):
+ *   Q block = 128 rows, K/V block = 64 rows; nq = ceil(N/128), nk = ceil(N/64).
+ */
+#ifndef SPARGEATTN_AMD_H
+#define SPARGEATTN_AMD_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+enum spg_status {
+  SPG_OK = 0,
+  SPG_ERR_INVALID = 1,      /* bad argument (maps to ValueError / RuntimeError on the Python side) */
+  SPG_ERR_UNSUPPORTED = 2,  /* valid but outside what the kernels cover (e.g. head_dim not in {64,128}) */
+  SPG_ERR_HIP = 3           /* a HIP runtime call failed */
+};
+
+enum spg_dtype { SPG_F16 = 0, SPG_BF16 = 1 };
+
+/* element kinds accepted for a user block mask ("non-zero = keep", spas_sage_attn/utils.py:68-69) */
+enum spg_mask_kind {
+  SPG_MASK_I8 = 0, SPG_MASK_I16 = 1, SPG_MASK_I32 = 2, SPG_MASK_I64 = 3,
+  SPG_MASK_F16 = 4, SPG_MASK_F32 = 5, SPG_MASK_F64 = 6   /* bf16 uses SPG_MASK_F16: both test (bits & 0x7fff) != 0 */
+};
+
+int spg_version(void);
+const char *spg_last_error(void);
+
+/* ---- A2: km = k.mean(dim=-2)  (spas_sage_attn/core.py:119-120) -------------------------------
+ * k (B,H,N,D) dtype -> km (B,H,D) dtype.  Column sums are accumulated in binary64 and rounded once.
+ * workspace: spg_km_mean_workspace_bytes() bytes of device scratch (per-chunk partial sums). */
+size_t spg_km_mean_workspace_bytes(int B, int H, int N, int D);
+int spg_km_mean(const void *k, void *km, void *workspace, int B, int H, int N, int D, int dtype, void *stream);
+
+/* ---- A3/A4: fused pool + self-similarity + per-block INT8 quantisation ------------------------
+ * replaces triton_bmm_pool_sim_simmean_fuse_quant (spas_sage_attn/utils.py:161-214, wrapper 270-280).
+ * x (B,H,N,D) dtype; km (B,H,D) dtype or NULL (Q: NULL, K: the column mean, subtracted in dtype);
+ * block = 128 (Q) or 64 (K); simthreshd1 (H,) float32.
+ * out: pool (B,H,nb,D) dtype; sim (B,H,nb) uint8 0/1; xq (B,H,N,D) int8; scale (B,H,nb) float32.
+ * ---- A13: with pool == NULL and sim == NULL this is qk_quantize (utils.py:89-159): xq and scale only. */
+int spg_pool_sim_quant(const void *x, const void *km, void *pool, uint8_t *sim, int8_t *xq, float *scale,
+                       const float *simthreshd1, int B, int H, int N, int D, int block, int dtype, void *stream);
+
+/* ---- A5-A8: compressed attention, top-k / CDF selection, block map, LUT ------------------------
+ * replaces the torch glue of get_block_map_meansim_fuse_quant (spas_sage_attn/utils.py:386-420),
+ * triton_fill_causal_mask (304-316), triton_fill_block_map_kernel (282-302) and
+ * triton_block_map_to_lut_kernel (54-87) with one kernel; the score matrix never reaches HBM.
+ * Exactly one of topk / cdfthreshd ((H,) float32 device pointers) is non-NULL.
+ * out: lut (B,H,nq,nk) int32 delta-encoded ascending block indices, zero tail;
+ *      valid_block_num (B,H,nq) int32; block_map (B,H,nq,nk) uint8 0/1 or NULL. */
+int spg_block_select(const void *pool_q, const uint8_t *sim_q, const void *pool_k, const uint8_t *sim_k,
+                     const float *topk, const float *cdfthreshd, int is_causal, int attention_sink,
+                     int32_t *lut, int32_t *valid_block_num, uint8_t *block_map,
+                     int B, int H, int nq, int nk, int D, int dtype, void *stream);
+
+/* ---- A8 alone: user block mask -> LUT  (block_map_lut_triton, spas_sage_attn/utils.py:76-87) ---- */
+int spg_map_to_lut(const void *mask, int mask_kind, int32_t *lut, int32_t *valid_block_num,
+                   int B, int H, int nq, int nk, void *stream);
+
+/* ---- A9+A10: V -> fp16 -> per-channel FP8 e4m3 ---------------------------------------------------
+ * replaces transpose_pad_permute_cuda + scale_fuse_quant_cuda(..., scale_max = 2.25)
+ * (csrc/fused/fused.cu:193-267, 269-344; called at core.py:147,151).
+ * v (B,H,N,D) dtype (bf16 input is first rounded to fp16, core.py:117).
+ * out: v8 e4m3fn codes in TILE layout [B][H][nk][D][64] (key index fastest inside a 64-key tile, rows
+ *      beyond N are zero) - the layout the attention kernel's V^T operand reads; v_scale (B,H,D) float32
+ *      = amax/2.25.  v_scale doubles as the amax scratch between the passes. */
+int spg_v_quant_fp8(const void *v, uint8_t *v8, float *v_scale, int B, int H, int N, int D, int dtype,
+                    void *stream);
+
+/* ---- A11: block-sparse INT8-QK / FP8-PV attention ------------------------------------------------
+ * replaces qk_int8_sv_f8_accum_f32_block_sparse_attn_inst_buf_fuse_v_scale_with_pv_threshold
+ * (csrc/qattn/attn_cuda.h:61-76, csrc/qattn/qk_int_sv_f8_cuda_sm89.cu:197-390) with
+ * tensor_layout = HND, qk_quant_gran = per-block, PV threshold per block.
+ * q8,k8 int8 (B,H,N,D); v8 as produced by spg_v_quant_fp8; out (B,H,N,D) out_dtype;
+ * lut/valid_block_num as above; pvthreshd (H,) float32; q_scale (B,H,nq), k_scale (B,H,nk),
+ * v_scale (B,H,D) float32; pv_count (B,H,nq) int32 or NULL (number of K blocks whose PV was computed).
+ * Row blocks with valid_block_num == 0 are left unwritten, as in the reference (sm89.cuh:232-235). */
+int spg_block_sparse_attn(const int8_t *q8, const int8_t *k8, const uint8_t *v8, void *out, int out_dtype,
+                          const int32_t *lut, const int32_t *valid_block_num, const float *pvthreshd,
+                          const float *q_scale, const float *k_scale, const float *v_scale,
+                          int B, int H, int N, int D, float sm_scale, int is_causal, int32_t *pv_count,
+                          void *stream);
+
+/* ---- measurement comparator: dense FP16 flash attention on MFMA (no counterpart in the reference;
+ * the "dense FP16 attention kernel built in the same run" the speed-up is quoted against).
+ * q,k,v,out (B,H,N,D) fp16. */
+int spg_dense_attn_f16(const void *q, const void *k, const void *v, void *out, int B, int H, int N, int D,
+                       float sm_scale, int is_causal, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* SPARGEATTN_AMD_H */

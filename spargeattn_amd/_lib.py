@@ -1,0 +1,195 @@
+"""ctypes binding of libspargeattn_amd.so (the C ABI in include/spargeattn_amd.h).
+
+PyTorch is used for device memory and streams only: every wrapper below hands raw
+``data_ptr()`` addresses and the current HIP stream to the library.  There is no CPU or
+eager fallback: if the library is missing, or no GPU tensor is given, the call raises.
+"""
+import ctypes
+import os
+
+import torch
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libspargeattn_amd.so")
+
+SPG_OK, SPG_ERR_INVALID, SPG_ERR_UNSUPPORTED, SPG_ERR_HIP = 0, 1, 2, 3
+SPG_F16, SPG_BF16 = 0, 1
+
+_c = ctypes
+_vp, _i, _f, _sz = _c.c_void_p, _c.c_int, _c.c_float, _c.c_size_t
+
+# symbol -> (restype, argtypes); must list every function include/spargeattn_amd.h declares
+SIGNATURES = {
+    "spg_version": (_i, []),
+    "spg_last_error": (_c.c_char_p, []),
+    "spg_km_mean_workspace_bytes": (_sz, [_i, _i, _i, _i]),
+    "spg_km_mean": (_i, [_vp, _vp, _vp, _i, _i, _i, _i, _i, _vp]),
+    "spg_pool_sim_quant": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp]),
+    "spg_block_select": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp]),
+    "spg_map_to_lut": (_i, [_vp, _i, _vp, _vp, _i, _i, _i, _i, _vp]),
+    "spg_v_quant_fp8": (_i, [_vp, _vp, _vp, _i, _i, _i, _i, _i, _vp]),
+    "spg_block_sparse_attn": (_i, [_vp, _vp, _vp, _vp, _i, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _f, _i, _vp, _vp]),
+    "spg_dense_attn_f16": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _f, _i, _vp]),
+}
+
+_lib = None
+
+
+class SpargeError(RuntimeError):
+    pass
+
+
+def load():
+    """Load the shared library (once).  Raises if it has not been built."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise SpargeError(
+                f"{LIB_PATH} not found: build it with `python -m spargeattn_amd.build` (hipcc, gfx950). "
+                "There is no fallback path.")
+        lib = ctypes.CDLL(LIB_PATH)
+        for name, (res, args) in SIGNATURES.items():
+            fn = getattr(lib, name)
+            fn.restype, fn.argtypes = res, args
+        _lib = lib
+    return _lib
+
+
+def _check(rc):
+    if rc == SPG_OK:
+        return
+    msg = load().spg_last_error().decode()
+    if rc in (SPG_ERR_INVALID, SPG_ERR_UNSUPPORTED):
+        raise ValueError(msg)
+    raise SpargeError(msg)
+
+
+def _dt(t):
+    if t.dtype == torch.float16:
+        return SPG_F16
+    if t.dtype == torch.bfloat16:
+        return SPG_BF16
+    raise RuntimeError(f"expected a float16 or bfloat16 tensor, got {t.dtype}")
+
+
+def _dev(*ts):
+    for t in ts:
+        if t is None:
+            continue
+        if not t.is_cuda:
+            raise RuntimeError("spargeattn_amd kernels need GPU tensors (there is no CPU path)")
+        if not t.is_contiguous():
+            raise RuntimeError("tensor must be contiguous")
+
+
+def _p(t):
+    return None if t is None else t.data_ptr()
+
+
+def _stream():
+    return torch.cuda.current_stream().cuda_stream
+
+
+_MASK_KIND = {
+    torch.bool: 0, torch.uint8: 0, torch.int8: 0, torch.int16: 1, torch.int32: 2, torch.int64: 3,
+    torch.float16: 4, torch.bfloat16: 4, torch.float32: 5, torch.float64: 6,
+}
+
+
+# ----------------------------------------------------------------------------------------------
+# stage wrappers (allocate outputs with torch, call the C ABI)
+# ----------------------------------------------------------------------------------------------
+
+def km_mean(k):
+    """k (B,H,N,D) -> km (B,H,1,D), same dtype."""
+    _dev(k)
+    B, H, N, D = k.shape
+    lib = load()
+    km = torch.empty((B, H, 1, D), dtype=k.dtype, device=k.device)
+    ws = torch.empty(max(1, lib.spg_km_mean_workspace_bytes(B, H, N, D)), dtype=torch.uint8, device=k.device)
+    _check(lib.spg_km_mean(_p(k), _p(km), _p(ws), B, H, N, D, _dt(k), _stream()))
+    return km
+
+
+def pool_sim_quant(x, km, block, simthreshd1=None, with_pool=True):
+    """Returns (pool, sim, x_int8, scale) - pool and sim are None when with_pool is False."""
+    _dev(x, km, simthreshd1)
+    B, H, N, D = x.shape
+    nb = (N + block - 1) // block
+    xq = torch.empty((B, H, N, D), dtype=torch.int8, device=x.device)
+    scale = torch.empty((B, H, nb), dtype=torch.float32, device=x.device)
+    pool = sim = None
+    if with_pool:
+        pool = torch.empty((B, H, nb, D), dtype=x.dtype, device=x.device)
+        sim = torch.empty((B, H, nb), dtype=torch.bool, device=x.device)
+    _check(load().spg_pool_sim_quant(_p(x), _p(km), _p(pool), _p(sim), _p(xq), _p(scale), _p(simthreshd1),
+                                     B, H, N, D, block, _dt(x), _stream()))
+    return pool, sim, xq, scale
+
+
+def block_select(pool_q, sim_q, pool_k, sim_k, topk=None, cdfthreshd=None, is_causal=False,
+                 attention_sink=False, return_map=False):
+    _dev(pool_q, sim_q, pool_k, sim_k, topk, cdfthreshd)
+    B, H, nq, D = pool_q.shape
+    nk = pool_k.shape[2]
+    lut = torch.empty((B, H, nq, nk), dtype=torch.int32, device=pool_q.device)
+    valid = torch.empty((B, H, nq), dtype=torch.int32, device=pool_q.device)
+    bmap = torch.empty((B, H, nq, nk), dtype=torch.bool, device=pool_q.device) if return_map else None
+    _check(load().spg_block_select(_p(pool_q), _p(sim_q), _p(pool_k), _p(sim_k), _p(topk), _p(cdfthreshd),
+                                   int(bool(is_causal)), int(bool(attention_sink)), _p(lut), _p(valid), _p(bmap),
+                                   B, H, nq, nk, D, _dt(pool_q), _stream()))
+    return lut, valid, bmap
+
+
+def map_to_lut(block_map):
+    _dev(block_map)
+    if block_map.dtype not in _MASK_KIND:
+        raise RuntimeError(f"unsupported mask dtype {block_map.dtype}")
+    B, H, nq, nk = block_map.shape
+    lut = torch.empty((B, H, nq, nk), dtype=torch.int32, device=block_map.device)
+    valid = torch.empty((B, H, nq), dtype=torch.int32, device=block_map.device)
+    _check(load().spg_map_to_lut(_p(block_map), _MASK_KIND[block_map.dtype], _p(lut), _p(valid), B, H, nq, nk, _stream()))
+    return lut, valid
+
+
+def v_quant_fp8(v):
+    """v (B,H,N,D) fp16/bf16 -> (v8 uint8 codes in tile layout (B,H,nk,D,64), v_scale (B,H,D) float32)."""
+    _dev(v)
+    B, H, N, D = v.shape
+    nk = (N + 63) // 64
+    v8 = torch.empty((B, H, nk, D, 64), dtype=torch.uint8, device=v.device)
+    v_scale = torch.empty((B, H, D), dtype=torch.float32, device=v.device)
+    _check(load().spg_v_quant_fp8(_p(v), _p(v8), _p(v_scale), B, H, N, D, _dt(v), _stream()))
+    return v8, v_scale
+
+
+def block_sparse_attn(q8, k8, v8, out, lut, valid, pvthreshd, q_scale, k_scale, v_scale, sm_scale,
+                      is_causal=False, return_pv_count=False):
+    _dev(q8, k8, v8, out, lut, valid, pvthreshd, q_scale, k_scale, v_scale)
+    B, H, N, D = q8.shape
+    pvc = torch.zeros((B, H, (N + 127) // 128), dtype=torch.int32, device=q8.device) if return_pv_count else None
+    _check(load().spg_block_sparse_attn(_p(q8), _p(k8), _p(v8), _p(out), _dt(out), _p(lut), _p(valid), _p(pvthreshd),
+                                        _p(q_scale), _p(k_scale), _p(v_scale), B, H, N, D, float(sm_scale),
+                                        int(bool(is_causal)), _p(pvc), _stream()))
+    return pvc
+
+
+def v_tiles_f16(v):
+    """(B,H,N,D) fp16 -> zero-padded (B,H,nk,D,64) tiles, the V^T layout the dense comparator reads."""
+    B, H, N, D = v.shape
+    nk = (N + 63) // 64
+    if nk * 64 != N:
+        v = torch.nn.functional.pad(v, (0, 0, 0, nk * 64 - N))
+    return v.view(B, H, nk, 64, D).transpose(-1, -2).contiguous()
+
+
+def dense_attn_f16(q, k, vt, sm_scale, is_causal=False, out=None):
+    """Dense fp16 flash attention (measurement comparator).  vt = v_tiles_f16(v)."""
+    _dev(q, k, vt)
+    assert q.dtype == k.dtype == vt.dtype == torch.float16
+    B, H, N, D = q.shape
+    if out is None:
+        out = torch.empty_like(q)
+    _check(load().spg_dense_attn_f16(_p(q), _p(k), _p(vt), _p(out), B, H, N, D, float(sm_scale),
+                                     int(bool(is_causal)), _stream()))
+    return out

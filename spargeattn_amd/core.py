@@ -1,0 +1,123 @@
+"""Operator API: drop-in for ``spas_sage_attn.core`` of thu-ml/SpargeAttn on MI355X.
+
+    spas_sage2_attn_meansim_topk_cuda   spas_sage_attn/core.py:105-169
+    spas_sage2_attn_meansim_cuda        spas_sage_attn/core.py:39-103   (CDF selection)
+    block_sparse_sage2_attn_cuda        spas_sage_attn/core.py:171-233
+
+Same names, argument order, defaults and return values.  The ``_cuda`` suffix is kept so that
+callers need no change; everything runs as HIP kernels for gfx950.  As in the reference,
+``attn_mask``, ``dropout_p`` and ``output_dtype`` are accepted and ignored, the output dtype is
+fp16 for fp32/fp16 inputs and bf16 for bf16 inputs, and causality is enforced at 128x64-block
+granularity through the LUT (the reference passes ``is_causal=False`` to its kernel, core.py:154-158).
+``kernel_causal=True`` is an extension that additionally masks at token level.
+"""
+import torch
+
+from . import _lib
+from .utils import (hyperparameter_check, get_block_map_meansim_fuse_quant, get_vanilla_qk_quant,
+                    block_map_lut_triton)
+
+
+# Optional callable(name) invoked at stage boundaries ("km", "maskpred", "vquant", "attn", "end");
+# bench.py installs one that records HIP events on the current stream.  None in normal use.
+_stage_hook = None
+
+
+def _mark(name):
+    if _stage_hook is not None:
+        _stage_hook(name)
+
+
+def _prologue(q, k, v, tensor_layout):
+    assert tensor_layout in ['HND', 'NHD']
+    if tensor_layout == 'NHD':
+        q, k, v = (t.transpose(-2, -3) for t in (q, k, v))
+    assert q.size(-2) >= 128, "seq_len should be not less than 128."
+    assert q.size(-1) in [64, 128], "headdim should be in [64, 128]. For other headdim, you can use padding and specify the softmax scale."
+    if not v.is_cuda:
+        raise RuntimeError("spargeattn_amd needs GPU tensors (there is no CPU path)")
+    torch.cuda.set_device(v.device)
+    qk_dtype = torch.bfloat16 if q.dtype == torch.bfloat16 else torch.float16
+    q = q.contiguous().to(qk_dtype)
+    k = k.contiguous().to(qk_dtype)
+    v = v.contiguous().to(torch.float16)       # V is always quantised from fp16 (core.py:117)
+    return q, k, v
+
+
+def _attention(q, k, v, q_int8, q_scale, k_int8, k_scale, lut, valid_block_num, scale, pvthreshd, kernel_causal,
+               return_pv_count=False):
+    headdim = q.size(-1)
+    if scale is None:
+        scale = 1.0 / (headdim ** 0.5)
+    assert headdim in [64, 128], "headdim should be in [64, 128]. For other headdim, you can use padding and specify the softmax scale."
+    pvthreshd = hyperparameter_check(pvthreshd, q.size(-3), q.device)
+    o = torch.empty_like(q)
+    _mark("vquant")
+    v_fp8, v_scale = _lib.v_quant_fp8(v)
+    _mark("attn")
+    pvc = _lib.block_sparse_attn(q_int8, k_int8, v_fp8, o, lut, valid_block_num, pvthreshd, q_scale, k_scale, v_scale,
+                                 scale, is_causal=kernel_causal, return_pv_count=return_pv_count)
+    _mark("end")
+    return o, pvc
+
+
+def _finish(o, tensor_layout, return_sparsity, valid_block_num, lut, causal_denominator):
+    if tensor_layout == 'NHD':
+        o = o.transpose(-2, -3)
+    if return_sparsity:
+        nq, nk = lut.size(2), lut.size(3)
+        cols = (nk + 2) // 2 if causal_denominator else nk
+        qk_sparsity = 1 - (valid_block_num.float().sum()) / (cols * nq * lut.size(0) * lut.size(1))
+        return o, qk_sparsity.item()
+    return o
+
+
+def _meansim(q, k, v, is_causal, scale, smooth_k, simthreshd1, cdfthreshd, topk, pvthreshd, attention_sink,
+             tensor_layout, return_sparsity, kernel_causal):
+    q, k, v = _prologue(q, k, v, tensor_layout)
+    if not smooth_k:
+        # the reference leaves `km` undefined in this case (core.py:119-126)
+        raise NameError("name 'km' is not defined")
+    _mark("km")
+    km = _lib.km_mean(k)
+    _mark("maskpred")
+    lut, valid_block_num, q_int8, q_scale, k_int8, k_scale = get_block_map_meansim_fuse_quant(
+        q, k, km, is_causal=is_causal, simthreshd1=simthreshd1, cdfthreshd=cdfthreshd, topk=topk, return_lut=True,
+        attention_sink=attention_sink, BLKQ=128, BLKK=64)
+    o, _ = _attention(q, k, v, q_int8, q_scale, k_int8, k_scale, lut, valid_block_num, scale, pvthreshd, kernel_causal)
+    return _finish(o, tensor_layout, return_sparsity, valid_block_num, lut, causal_denominator=is_causal is not False)
+
+
+@torch.compiler.disable
+def spas_sage2_attn_meansim_cuda(q, k, v, attn_mask=None, dropout_p=0.0, is_causal=False, scale=None, smooth_k=True,
+                                 simthreshd1=0.6, cdfthreshd=0.98, pvthreshd=50, attention_sink=False,
+                                 tensor_layout="HND", output_dtype=torch.float16, return_sparsity=False,
+                                 kernel_causal=False):
+    return _meansim(q, k, v, is_causal, scale, smooth_k, simthreshd1, cdfthreshd, None, pvthreshd, attention_sink,
+                    tensor_layout, return_sparsity, kernel_causal)
+
+
+@torch.compiler.disable
+def spas_sage2_attn_meansim_topk_cuda(q, k, v, attn_mask=None, dropout_p=0.0, is_causal=False, scale=None,
+                                      smooth_k=True, simthreshd1=-0.1, cdfthreshd=None, topk=0.5, pvthreshd=50,
+                                      attention_sink=False, tensor_layout="HND", output_dtype=torch.float16,
+                                      return_sparsity=False, kernel_causal=False):
+    return _meansim(q, k, v, is_causal, scale, smooth_k, simthreshd1, cdfthreshd, topk, pvthreshd, attention_sink,
+                    tensor_layout, return_sparsity, kernel_causal)
+
+
+@torch.compiler.disable
+def block_sparse_sage2_attn_cuda(q, k, v, mask_id=None, dropout_p=0.0, scale=None, smooth_k=True, pvthreshd=50,
+                                 attention_sink=False, tensor_layout="HND", output_dtype=torch.float16,
+                                 return_sparsity=False, kernel_causal=False):
+    q, k, v = _prologue(q, k, v, tensor_layout)
+    if not smooth_k:
+        raise NameError("name 'km' is not defined")
+    _mark("km")
+    km = _lib.km_mean(k)
+    _mark("maskpred")
+    q_int8, q_scale, k_int8, k_scale = get_vanilla_qk_quant(q, k, km, 128, 64)
+    lut, valid_block_num = block_map_lut_triton(block_map=mask_id)
+    o, _ = _attention(q, k, v, q_int8, q_scale, k_int8, k_scale, lut, valid_block_num, scale, pvthreshd, kernel_causal)
+    # the reference always reports against the causal denominator here (core.py:230)
+    return _finish(o, tensor_layout, return_sparsity, valid_block_num, lut, causal_denominator=True)

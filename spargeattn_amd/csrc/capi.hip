@@ -1,0 +1,138 @@
+// extern "C" entry points declared in include/spargeattn_amd.h: argument checks, then a launch on the caller's
+// stream.  No allocation, no synchronisation, no global state (the error string is thread-local).
+#include "../../include/spargeattn_amd.h"
+#include "launch.h"
+
+#include <cstdarg>
+#include <cstdio>
+
+namespace {
+thread_local char g_err[512] = "";
+
+int fail(int code, const char *fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_err, sizeof(g_err), fmt, ap);
+  va_end(ap);
+  return code;
+}
+
+int check_launch(const char *what, hipError_t e) {
+  if (e == hipSuccess) e = hipGetLastError();
+  if (e != hipSuccess) return fail(SPG_ERR_HIP, "%s: %s", what, hipGetErrorString(e));
+  return SPG_OK;
+}
+
+int check_shape(const char *fn, int B, int H, int N, int D) {
+  if (B <= 0 || H <= 0 || N <= 0) return fail(SPG_ERR_INVALID, "%s: B, H, N must be positive (got %d, %d, %d)", fn, B, H, N);
+  if (D != 64 && D != 128) return fail(SPG_ERR_UNSUPPORTED, "%s: head_dim must be 64 or 128 (got %d)", fn, D);
+  if ((double)B * H * (double)N * D >= 4294967296.0 * 4)
+    return fail(SPG_ERR_UNSUPPORTED, "%s: tensor too large (B*H*N*D = %.0f)", fn, (double)B * H * (double)N * D);
+  return SPG_OK;
+}
+
+int check_dtype(const char *fn, int dtype) {
+  if (dtype != SPG_F16 && dtype != SPG_BF16) return fail(SPG_ERR_INVALID, "%s: dtype must be SPG_F16 or SPG_BF16 (got %d)", fn, dtype);
+  return SPG_OK;
+}
+
+#define SPG_TRY(expr) do { int rc_ = (expr); if (rc_ != SPG_OK) return rc_; } while (0)
+#define SPG_NONNULL(fn, ptr) do { if ((ptr) == nullptr) return fail(SPG_ERR_INVALID, "%s: %s is NULL", fn, #ptr); } while (0)
+}  // namespace
+
+extern "C" {
+
+int spg_version(void) { return 100; }
+
+const char *spg_last_error(void) { return g_err; }
+
+size_t spg_km_mean_workspace_bytes(int B, int H, int N, int D) {
+  if (B <= 0 || H <= 0 || N <= 0 || D <= 0) return 0;
+  return spg::km_mean_workspace_bytes(B, H, N, D);
+}
+
+int spg_km_mean(const void *k, void *km, void *workspace, int B, int H, int N, int D, int dtype, void *stream) {
+  const char *fn = "spg_km_mean";
+  SPG_TRY(check_shape(fn, B, H, N, D));
+  SPG_TRY(check_dtype(fn, dtype));
+  SPG_NONNULL(fn, k); SPG_NONNULL(fn, km); SPG_NONNULL(fn, workspace);
+  spg::launch_km_mean(k, km, workspace, B, H, N, D, dtype, (hipStream_t)stream);
+  return check_launch(fn, hipSuccess);
+}
+
+int spg_pool_sim_quant(const void *x, const void *km, void *pool, uint8_t *sim, int8_t *xq, float *scale,
+                       const float *simthreshd1, int B, int H, int N, int D, int block, int dtype, void *stream) {
+  const char *fn = "spg_pool_sim_quant";
+  SPG_TRY(check_shape(fn, B, H, N, D));
+  SPG_TRY(check_dtype(fn, dtype));
+  if (block != 64 && block != 128) return fail(SPG_ERR_UNSUPPORTED, "%s: block must be 64 or 128 (got %d)", fn, block);
+  SPG_NONNULL(fn, x); SPG_NONNULL(fn, xq); SPG_NONNULL(fn, scale);
+  if ((pool == nullptr) != (sim == nullptr)) return fail(SPG_ERR_INVALID, "%s: pool and sim must both be given or both be NULL", fn);
+  if (pool != nullptr) SPG_NONNULL(fn, simthreshd1);
+  spg::launch_pool_sim_quant(x, km, pool, sim, xq, scale, simthreshd1, B, H, N, D, block, dtype, (hipStream_t)stream);
+  return check_launch(fn, hipSuccess);
+}
+
+int spg_block_select(const void *pool_q, const uint8_t *sim_q, const void *pool_k, const uint8_t *sim_k,
+                     const float *topk, const float *cdfthreshd, int is_causal, int attention_sink, int32_t *lut,
+                     int32_t *valid_block_num, uint8_t *block_map, int B, int H, int nq, int nk, int D, int dtype,
+                     void *stream) {
+  const char *fn = "spg_block_select";
+  if (B <= 0 || H <= 0 || nq <= 0 || nk <= 0) return fail(SPG_ERR_INVALID, "%s: B, H, nq, nk must be positive", fn);
+  if (D != 64 && D != 128) return fail(SPG_ERR_UNSUPPORTED, "%s: head_dim must be 64 or 128 (got %d)", fn, D);
+  SPG_TRY(check_dtype(fn, dtype));
+  if ((topk == nullptr) == (cdfthreshd == nullptr))
+    return fail(SPG_ERR_INVALID, "%s: Only one of cdfthreshd and topk can be set.", fn);
+  if (nk > spg::block_select_max_nk())
+    return fail(SPG_ERR_UNSUPPORTED, "%s: nk = %d exceeds the supported maximum %d", fn, nk, spg::block_select_max_nk());
+  SPG_NONNULL(fn, pool_q); SPG_NONNULL(fn, sim_q); SPG_NONNULL(fn, pool_k); SPG_NONNULL(fn, sim_k);
+  SPG_NONNULL(fn, lut); SPG_NONNULL(fn, valid_block_num);
+  return check_launch(fn, spg::launch_block_select(pool_q, sim_q, pool_k, sim_k, topk, cdfthreshd, is_causal ? 1 : 0,
+                                                   attention_sink ? 1 : 0, lut, valid_block_num, block_map, B, H, nq,
+                                                   nk, D, dtype, (hipStream_t)stream));
+}
+
+int spg_map_to_lut(const void *mask, int mask_kind, int32_t *lut, int32_t *valid_block_num, int B, int H, int nq,
+                   int nk, void *stream) {
+  const char *fn = "spg_map_to_lut";
+  if (B <= 0 || H <= 0 || nq <= 0 || nk <= 0) return fail(SPG_ERR_INVALID, "%s: B, H, nq, nk must be positive", fn);
+  if (mask_kind < SPG_MASK_I8 || mask_kind > SPG_MASK_F64) return fail(SPG_ERR_INVALID, "%s: bad mask_kind %d", fn, mask_kind);
+  if (nk > 32768) return fail(SPG_ERR_UNSUPPORTED, "%s: nk = %d exceeds the supported maximum 32768", fn, nk);
+  SPG_NONNULL(fn, mask); SPG_NONNULL(fn, lut); SPG_NONNULL(fn, valid_block_num);
+  return check_launch(fn, spg::launch_map_to_lut(mask, mask_kind, lut, valid_block_num, B, H, nq, nk, (hipStream_t)stream));
+}
+
+int spg_v_quant_fp8(const void *v, uint8_t *v8, float *v_scale, int B, int H, int N, int D, int dtype, void *stream) {
+  const char *fn = "spg_v_quant_fp8";
+  SPG_TRY(check_shape(fn, B, H, N, D));
+  SPG_TRY(check_dtype(fn, dtype));
+  SPG_NONNULL(fn, v); SPG_NONNULL(fn, v8); SPG_NONNULL(fn, v_scale);
+  spg::launch_v_quant_fp8(v, v8, v_scale, B, H, N, D, dtype, (hipStream_t)stream);
+  return check_launch(fn, hipSuccess);
+}
+
+int spg_block_sparse_attn(const int8_t *q8, const int8_t *k8, const uint8_t *v8, void *out, int out_dtype,
+                          const int32_t *lut, const int32_t *valid_block_num, const float *pvthreshd,
+                          const float *q_scale, const float *k_scale, const float *v_scale, int B, int H, int N, int D,
+                          float sm_scale, int is_causal, int32_t *pv_count, void *stream) {
+  const char *fn = "spg_block_sparse_attn";
+  SPG_TRY(check_shape(fn, B, H, N, D));
+  SPG_TRY(check_dtype(fn, out_dtype));
+  SPG_NONNULL(fn, q8); SPG_NONNULL(fn, k8); SPG_NONNULL(fn, v8); SPG_NONNULL(fn, out); SPG_NONNULL(fn, lut);
+  SPG_NONNULL(fn, valid_block_num); SPG_NONNULL(fn, pvthreshd); SPG_NONNULL(fn, q_scale); SPG_NONNULL(fn, k_scale);
+  SPG_NONNULL(fn, v_scale);
+  return check_launch(fn, spg::launch_block_sparse_attn(q8, k8, v8, out, out_dtype, lut, valid_block_num, pvthreshd,
+                                                        q_scale, k_scale, v_scale, B, H, N, D, sm_scale,
+                                                        is_causal ? 1 : 0, pv_count, (hipStream_t)stream));
+}
+
+int spg_dense_attn_f16(const void *q, const void *k, const void *v, void *out, int B, int H, int N, int D,
+                       float sm_scale, int is_causal, void *stream) {
+  const char *fn = "spg_dense_attn_f16";
+  SPG_TRY(check_shape(fn, B, H, N, D));
+  SPG_NONNULL(fn, q); SPG_NONNULL(fn, k); SPG_NONNULL(fn, v); SPG_NONNULL(fn, out);
+  return check_launch(fn, spg::launch_dense_attn_f16(q, k, v, out, B, H, N, D, sm_scale, is_causal ? 1 : 0,
+                                                     (hipStream_t)stream));
+}
+
+}  // extern "C"

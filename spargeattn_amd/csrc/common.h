@@ -1,0 +1,94 @@
+// Shared device helpers for the gfx950 SpargeAttn kernels: element conversions with a single rounding,
+// wavefront (64-lane) and workgroup reductions, error plumbing for the C ABI.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#define SPG_WAVE 64
+
+namespace spg {
+
+// ---------------------------------------------------------------------------------------------
+// 16-bit element types.  DT = 0: IEEE binary16, DT = 1: bfloat16 (same numbering as enum spg_dtype).
+// ---------------------------------------------------------------------------------------------
+template <int DT> __device__ __forceinline__ float elem_to_f32(uint16_t b);
+template <> __device__ __forceinline__ float elem_to_f32<0>(uint16_t b) {
+  _Float16 h = __builtin_bit_cast(_Float16, b);
+  return (float)h;
+}
+template <> __device__ __forceinline__ float elem_to_f32<1>(uint16_t b) {
+  return __builtin_bit_cast(float, (uint32_t)b << 16);
+}
+
+// binary64 -> 16-bit pattern with ONE round-to-nearest-even (never through binary32).
+// MANT mantissa bits, BIAS exponent bias, EMIN exponent of the smallest normal.
+template <int MANT, int BIAS, int EMIN>
+__device__ __forceinline__ uint16_t f64_to_bits16(double x) {
+  const uint64_t b = __builtin_bit_cast(uint64_t, x);
+  const uint16_t sign = (uint16_t)((b >> 63) << 15);
+  const uint64_t a = b & 0x7fffffffffffffffull;
+  const double ax = __builtin_bit_cast(double, a);
+  constexpr int EXPBITS = 15 - MANT;
+  constexpr uint16_t INF = (uint16_t)(((1u << EXPBITS) - 1u) << MANT);
+  if (a > 0x7ff0000000000000ull) return sign | INF | (uint16_t)(1u << (MANT - 1));  // NaN
+  // largest finite = (2 - 2^-MANT) * 2^(INFEXP-1-BIAS); halfway to the next binade rounds to inf
+  constexpr int EMAX = ((1 << EXPBITS) - 2) - BIAS;
+  const double ovf = __builtin_ldexp(2.0 - __builtin_ldexp(1.0, -MANT - 1), EMAX);
+  if (ax >= ovf) return sign | INF;
+  if (ax < __builtin_ldexp(1.0, EMIN)) {
+    const double y = __builtin_rint(ax * __builtin_ldexp(1.0, MANT - EMIN));  // count of subnormal quanta
+    return sign | (uint16_t)(int)y;
+  }
+  constexpr int SH = 52 - MANT;
+  const uint64_t lsb = (a >> SH) & 1ull;
+  const uint64_t r = (a + ((1ull << (SH - 1)) - 1ull) + lsb) >> SH;            // [exp11 | mant]
+  return sign | (uint16_t)(r - ((uint64_t)(1023 - BIAS) << MANT));
+}
+
+template <int DT> __device__ __forceinline__ uint16_t f64_to_elem(double x);
+template <> __device__ __forceinline__ uint16_t f64_to_elem<0>(double x) { return f64_to_bits16<10, 15, -14>(x); }
+template <> __device__ __forceinline__ uint16_t f64_to_elem<1>(double x) { return f64_to_bits16<7, 127, -126>(x); }
+
+// binary32 -> 16-bit pattern, RNE (used for outputs that are produced in fp32)
+template <int DT> __device__ __forceinline__ uint16_t f32_to_elem(float x);
+template <> __device__ __forceinline__ uint16_t f32_to_elem<0>(float x) {
+  _Float16 h = (_Float16)x;
+  return __builtin_bit_cast(uint16_t, h);
+}
+template <> __device__ __forceinline__ uint16_t f32_to_elem<1>(float x) {
+  uint32_t u = __builtin_bit_cast(uint32_t, x);
+  if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x40);
+  u += 0x7fffu + ((u >> 16) & 1u);
+  return (uint16_t)(u >> 16);
+}
+
+// ---------------------------------------------------------------------------------------------
+// wavefront shuffles for 64-bit values
+// ---------------------------------------------------------------------------------------------
+__device__ __forceinline__ double shfl_xor_f64(double v, int mask) {
+  uint64_t u = __builtin_bit_cast(uint64_t, v);
+  uint32_t lo = (uint32_t)u, hi = (uint32_t)(u >> 32);
+  lo = __shfl_xor(lo, mask, SPG_WAVE);
+  hi = __shfl_xor(hi, mask, SPG_WAVE);
+  return __builtin_bit_cast(double, ((uint64_t)hi << 32) | lo);
+}
+__device__ __forceinline__ long long shfl_xor_i64(long long v, int mask) {
+  uint64_t u = (uint64_t)v;
+  uint32_t lo = (uint32_t)u, hi = (uint32_t)(u >> 32);
+  lo = __shfl_xor(lo, mask, SPG_WAVE);
+  hi = __shfl_xor(hi, mask, SPG_WAVE);
+  return (long long)(((uint64_t)hi << 32) | lo);
+}
+
+__device__ __forceinline__ float wave_max_f32(float v) {
+#pragma unroll
+  for (int o = 32; o >= 1; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, SPG_WAVE));
+  return v;
+}
+__device__ __forceinline__ int wave_sum_i32(int v) {
+#pragma unroll
+  for (int o = 32; o >= 1; o >>= 1) v += __shfl_xor(v, o, SPG_WAVE);
+  return v;
+}
+
+}  // namespace spg

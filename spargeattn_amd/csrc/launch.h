@@ -1,0 +1,31 @@
+// Host-side launch functions shared between the kernel translation units and the C ABI (capi.hip).
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stddef.h>
+#include <stdint.h>
+
+namespace spg {
+
+size_t km_mean_workspace_bytes(int B, int H, int N, int D);
+void launch_km_mean(const void *k, void *km, void *ws, int B, int H, int N, int D, int dtype, hipStream_t st);
+void launch_pool_sim_quant(const void *x, const void *km, void *pool, uint8_t *sim, int8_t *xq, float *scale,
+                           const float *thr, int B, int H, int N, int D, int block, int dtype, hipStream_t st);
+int block_select_max_nk();
+hipError_t launch_block_select(const void *pq, const uint8_t *sq, const void *pk, const uint8_t *sk, const float *topk,
+                               const float *cdf, int causal, int sink, int32_t *lut, int32_t *valid, uint8_t *bmap,
+                               int B, int H, int nq, int nk, int D, int dtype, hipStream_t st);
+hipError_t launch_map_to_lut(const void *mask, int kind, int32_t *lut, int32_t *valid, int B, int H, int nq, int nk,
+                             hipStream_t st);
+
+void launch_v_quant_fp8(const void *v, uint8_t *v8, float *v_scale, int B, int H, int N, int D, int dtype,
+                        hipStream_t st);
+
+hipError_t launch_block_sparse_attn(const int8_t *q8, const int8_t *k8, const uint8_t *v8, void *out, int out_dtype,
+                                    const int32_t *lut, const int32_t *valid, const float *pvthreshd,
+                                    const float *q_scale, const float *k_scale, const float *v_scale, int B, int H,
+                                    int N, int D, float sm_scale, int is_causal, int32_t *pv_count, hipStream_t st);
+
+hipError_t launch_dense_attn_f16(const void *q, const void *k, const void *v, void *out, int B, int H, int N, int D,
+                                 float sm_scale, int is_causal, hipStream_t st);
+
+}  // namespace spg

@@ -1,0 +1,541 @@
+// Sparse-mask prediction and INT8 Q/K quantisation for gfx950.
+//
+// Kernels (all HBM-bandwidth bound; one 16-byte load per lane, 64-lane wavefront reductions):
+//   km_partial / km_final      K column mean                          (spas_sage_attn/core.py:119-120)
+//   pool_sim_quant             pool + self-similarity + INT8 quant    (spas_sage_attn/utils.py:161-214, 89-159)
+//   block_select               compressed QK^T softmax, top-k / CDF selection, block map, delta LUT
+//                                                                     (spas_sage_attn/utils.py:386-420, 54-87, 282-316)
+//   map_to_lut                 user block mask -> LUT                 (spas_sage_attn/utils.py:54-87)
+//
+// Arithmetic contract: reductions whose addends are exactly representable run in binary64 (exact, hence
+// order independent); every tensor the reference materialises in the input dtype is rounded exactly once
+// (round-to-nearest-even, straight from binary64); fp32 quantisation steps use IEEE divide / sqrt; the
+// compressed softmax uses a fixed binary64 operation sequence and a fixed summation tree.  This file must be
+// compiled with -ffp-contract=off.
+#include "common.h"
+#include "launch.h"
+
+namespace spg {
+
+// =============================================================================================
+// K column mean
+// =============================================================================================
+template <int D, int DT>
+__global__ __launch_bounds__(256) void km_partial_kernel(const uint16_t *__restrict__ k, double *__restrict__ part,
+                                                         int N, int rows_per_chunk) {
+  constexpr int TPR = D / 8;      // lanes per row (16 B each)
+  constexpr int RPP = 256 / TPR;  // rows per pass of the workgroup
+  const int bh = blockIdx.y, chunk = blockIdx.x, nchunk = gridDim.x;
+  const int c = threadIdx.x % TPR, r = threadIdx.x / TPR;
+  const int row0 = chunk * rows_per_chunk;
+  const int row1 = min(N, row0 + rows_per_chunk);
+  const uint16_t *base = k + (size_t)bh * N * D + c * 8;
+  double acc[8];
+#pragma unroll
+  for (int e = 0; e < 8; e++) acc[e] = 0.0;
+#pragma unroll 4
+  for (int row = row0 + r; row < row1; row += RPP) {
+    const uint4 v = *(const uint4 *)(base + (size_t)row * D);
+    const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+    for (int e = 0; e < 4; e++) {
+      acc[2 * e] += (double)elem_to_f32<DT>((uint16_t)(w[e] & 0xffffu));
+      acc[2 * e + 1] += (double)elem_to_f32<DT>((uint16_t)(w[e] >> 16));
+    }
+  }
+  __shared__ double sm[RPP][D];
+#pragma unroll
+  for (int e = 0; e < 8; e++) sm[r][c * 8 + e] = acc[e];
+  __syncthreads();
+  if (threadIdx.x < D) {
+    double s = 0.0;
+    for (int i = 0; i < RPP; i++) s += sm[i][threadIdx.x];
+    part[((size_t)bh * nchunk + chunk) * D + threadIdx.x] = s;
+  }
+}
+
+template <int DT>
+__global__ void km_final_kernel(const double *__restrict__ part, uint16_t *__restrict__ km, int nchunk, int D, int N) {
+  const int bh = blockIdx.x, d = threadIdx.x;
+  double s = 0.0;
+  for (int i = 0; i < nchunk; i++) s += part[((size_t)bh * nchunk + i) * D + d];
+  km[(size_t)bh * D + d] = f64_to_elem<DT>(s / (double)N);
+}
+
+// =============================================================================================
+// pool + sim + INT8 quantisation.  One workgroup per (block, b*h).
+// =============================================================================================
+template <int BS, int D, int DT, bool HAS_MEAN, bool WITH_POOL>
+__global__ __launch_bounds__(256) void pool_sim_quant_kernel(const uint16_t *__restrict__ x,
+                                                             const uint16_t *__restrict__ km,
+                                                             uint16_t *__restrict__ pool, uint8_t *__restrict__ sim,
+                                                             int8_t *__restrict__ xq, float *__restrict__ scale,
+                                                             const float *__restrict__ simthr, int H, int N, int nb) {
+  constexpr int TPR = D / 8;
+  constexpr int RPP = 256 / TPR;
+  constexpr int NP = BS / RPP;
+  const int blk = blockIdx.x, bh = blockIdx.y;
+  const int tid = threadIdx.x, c = tid % TPR, r = tid / TPR;
+  const int row_base = blk * BS;
+  const int rows_valid = min(BS, N - row_base);
+  const uint16_t *xb = x + ((size_t)bh * N + row_base) * D + c * 8;
+
+  float kmf[8];
+  if constexpr (HAS_MEAN) {
+    const uint4 v = *(const uint4 *)(km + (size_t)bh * D + c * 8);
+    const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+    for (int e = 0; e < 4; e++) {
+      kmf[2 * e] = elem_to_f32<DT>((uint16_t)(w[e] & 0xffffu));
+      kmf[2 * e + 1] = elem_to_f32<DT>((uint16_t)(w[e] >> 16));
+    }
+  }
+
+  float xf[NP][8];
+  float amax = 0.f;
+#pragma unroll
+  for (int p = 0; p < NP; p++) {
+    const int row = r + p * RPP;
+    const bool ok = row < rows_valid;
+    uint4 v = make_uint4(0, 0, 0, 0);
+    if (ok) v = *(const uint4 *)(xb + (size_t)row * D);
+    const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+    for (int e = 0; e < 8; e++) {
+      float f = elem_to_f32<DT>((uint16_t)((e & 1) ? (w[e >> 1] >> 16) : (w[e >> 1] & 0xffffu)));
+      if constexpr (HAS_MEAN) {
+        // (k - km) rounded once to the input dtype; masked rows stay zero (utils.py:184-188)
+        if (ok) f = elem_to_f32<DT>(f64_to_elem<DT>((double)f - (double)kmf[e]));
+      }
+      xf[p][e] = f;
+      amax = fmaxf(amax, fabsf(f));
+    }
+  }
+
+  __shared__ float s_wmax[4];
+  __shared__ long long s_wg[4];
+  amax = wave_max_f32(amax);
+  if ((tid & 63) == 0) s_wmax[tid >> 6] = amax;
+
+  if constexpr (WITH_POOL) {
+    __shared__ double s_col[RPP][D];
+    __shared__ long long s_xi[RPP][D];
+    double colsum[8];
+    long long colxi[8];
+#pragma unroll
+    for (int e = 0; e < 8; e++) { colsum[e] = 0.0; colxi[e] = 0; }
+    int bad = 0;
+#pragma unroll
+    for (int p = 0; p < NP; p++) {
+      double ss = 0.0;
+#pragma unroll
+      for (int e = 0; e < 8; e++) {
+        const double xd = (double)xf[p][e];
+        ss += xd * xd;
+        colsum[e] += xd;
+      }
+#pragma unroll
+      for (int o = TPR / 2; o >= 1; o >>= 1) ss += shfl_xor_f64(ss, o);
+      const float norm = sqrtf((float)ss);
+#pragma unroll
+      for (int e = 0; e < 8; e++) {
+        const float xh = xf[p][e] / norm;          // 0/0 -> NaN for all-zero (masked) rows
+        const _Float16 h = (_Float16)xh;
+        const float hf = (float)h;
+        if (__builtin_isfinite(hf)) colxi[e] += (long long)(int)(hf * 16777216.0f);  // exact: fp16 = int * 2^-24
+        else bad = 1;
+      }
+    }
+#pragma unroll
+    for (int e = 0; e < 8; e++) { s_col[r][c * 8 + e] = colsum[e]; s_xi[r][c * 8 + e] = colxi[e]; }
+    const int any_bad = __syncthreads_or(bad);
+    long long g = 0;
+    if (tid < D) {
+      double s = 0.0;
+      long long sx = 0;
+      for (int i = 0; i < RPP; i++) { s += s_col[i][tid]; sx += s_xi[i][tid]; }
+      pool[((size_t)bh * nb + blk) * D + tid] = f64_to_elem<DT>(s / (double)rows_valid);
+      g = sx * sx;
+    }
+#pragma unroll
+    for (int o = 32; o >= 1; o >>= 1) g += shfl_xor_i64(g, o);
+    if ((tid & 63) == 0) s_wg[tid >> 6] = g;
+    __syncthreads();
+    if (tid == 0) {
+      const long long gt = s_wg[0] + s_wg[1] + s_wg[2] + s_wg[3];   // = sum(gram) * 2^48, exact
+      const double thr = (double)simthr[bh % H] * (double)(rows_valid * rows_valid) * 281474976710656.0;
+      sim[(size_t)bh * nb + blk] = (!any_bad && (double)gt > thr) ? 1 : 0;
+    }
+  } else {
+    __syncthreads();
+  }
+
+  amax = fmaxf(fmaxf(s_wmax[0], s_wmax[1]), fmaxf(s_wmax[2], s_wmax[3]));
+  const float s = amax / 127.0f + 1e-7f;
+  int8_t *qb = xq + ((size_t)bh * N + row_base) * D + c * 8;
+#pragma unroll
+  for (int p = 0; p < NP; p++) {
+    const int row = r + p * RPP;
+    if (row < rows_valid) {
+      uint32_t pk[2] = {0, 0};
+#pragma unroll
+      for (int e = 0; e < 8; e++) {
+        float y = xf[p][e] / s;
+        y = y + (y >= 0.f ? 0.5f : -0.5f);
+        const int q = (int)y;   // truncation toward zero
+        pk[e >> 2] |= ((uint32_t)q & 0xffu) << (8 * (e & 3));
+      }
+      *(uint2 *)(qb + (size_t)row * D) = make_uint2(pk[0], pk[1]);
+    }
+  }
+  if (tid == 0) scale[(size_t)bh * nb + blk] = s;
+}
+
+// =============================================================================================
+// canonical exp: a fixed sequence of binary64 mul / add (no fma), t <= 0.
+// =============================================================================================
+__device__ __forceinline__ double cexp(double t) {
+  if (!(t >= -700.0)) return 0.0;
+  const double k = __builtin_rint(t * 1.4426950408889634);
+  const double r = (t - k * 0.6931471803691238) - k * 1.9082149292705877e-10;
+  double p = 1.0 / 6227020800.0;
+  p = p * r; p = p + 1.0 / 479001600.0;
+  p = p * r; p = p + 1.0 / 39916800.0;
+  p = p * r; p = p + 1.0 / 3628800.0;
+  p = p * r; p = p + 1.0 / 362880.0;
+  p = p * r; p = p + 1.0 / 40320.0;
+  p = p * r; p = p + 1.0 / 5040.0;
+  p = p * r; p = p + 1.0 / 720.0;
+  p = p * r; p = p + 1.0 / 120.0;
+  p = p * r; p = p + 1.0 / 24.0;
+  p = p * r; p = p + 1.0 / 6.0;
+  p = p * r; p = p + 1.0 / 2.0;
+  p = p * r; p = p + 1.0;
+  p = p * r; p = p + 1.0;
+  return __builtin_ldexp(p, (int)k);
+}
+
+// exclusive prefix of per-thread counts over the 256 threads of the workgroup; returns (offset, total)
+__device__ __forceinline__ int2 block_exclusive_scan_i32(int v, int *s_tmp /* >= 256 ints */) {
+  const int tid = threadIdx.x;
+  s_tmp[tid] = v;
+  __syncthreads();
+  int off = 0, tot = 0;
+  for (int u = 0; u < 256; u++) {
+    const int w = s_tmp[u];
+    off += (u < tid) ? w : 0;
+    tot += w;
+  }
+  __syncthreads();
+  return make_int2(off, tot);
+}
+
+// flags (per column, via functor) -> ascending compact index list -> delta LUT, zero tail, valid count.
+template <class FlagFn>
+__device__ __forceinline__ void emit_lut(FlagFn flag, int nk, int nkp, int32_t *s_idx, int *s_tmp,
+                                         int32_t *__restrict__ lut_row, int32_t *__restrict__ valid_out) {
+  const int tid = threadIdx.x;
+  const int seg = nkp / 256;
+  const int j0 = tid * seg, j1 = min(nk, j0 + seg);
+  int cnt = 0;
+  for (int j = j0; j < j1; j++) cnt += flag(j) ? 1 : 0;
+  const int2 st = block_exclusive_scan_i32(cnt, s_tmp);
+  int pos = st.x;
+  for (int j = j0; j < j1; j++)
+    if (flag(j)) s_idx[pos++] = j;
+  __syncthreads();
+  for (int p = tid; p < nk; p += 256) {
+    int v = 0;
+    if (p < st.y) v = s_idx[p] - (p ? s_idx[p - 1] : 0);
+    lut_row[p] = v;
+  }
+  if (tid == 0) *valid_out = st.y;
+}
+
+// =============================================================================================
+// block_select: one workgroup per (q block row, b*h).
+// dynamic LDS: 12 * nkp bytes (nkp = power of two >= max(nk, 256)).
+// =============================================================================================
+template <int D, int DT>
+__global__ __launch_bounds__(256) void block_select_kernel(
+    const uint16_t *__restrict__ pool_q, const uint8_t *__restrict__ sim_q, const uint16_t *__restrict__ pool_k,
+    const uint8_t *__restrict__ sim_k, const float *__restrict__ topk, const float *__restrict__ cdfthr, int is_causal,
+    int sink, int32_t *__restrict__ lut, int32_t *__restrict__ valid, uint8_t *__restrict__ bmap, int H, int nq, int nk,
+    int nkp) {
+  extern __shared__ __align__(16) unsigned char smem[];
+  double *e_buf = (double *)smem;                    // [nkp] exp values        (phase 1)
+  uint32_t *skey = (uint32_t *)smem;                 // [nkp] sorted keys       (phase 2, aliases e_buf)
+  int32_t *s_idx = (int32_t *)(smem + 4 * (size_t)nkp);  // [nkp] compact indices (phase 3, aliases e_buf)
+  uint32_t *okey = (uint32_t *)(smem + 8 * (size_t)nkp); // [nkp] scores, then keys in column order
+  __shared__ float s_pq[D];
+  __shared__ float s_wmax[4];
+  __shared__ double s_wsum[4];
+  __shared__ double s_tsum[256];
+  __shared__ int s_tmp[256];
+  __shared__ int s_n;
+
+  const int i = blockIdx.x, bh = blockIdx.y, h = bh % H, tid = threadIdx.x;
+  if (tid < D) s_pq[tid] = elem_to_f32<DT>(pool_q[((size_t)bh * nq + i) * D + tid]);
+  __syncthreads();
+
+  const float sm_scale = (D == 64) ? 0.125f : 0.088388347648318447f;  // fp32(D^-0.5)
+  const int causal_lim = is_causal ? min(nk, 2 * (i + 1)) : nk;
+  const uint16_t *pk_base = pool_k + (size_t)bh * nk * D;
+  const uint8_t *simk = sim_k + (size_t)bh * nk;
+  float *s_score = (float *)okey;
+
+  // ---- scores (fixed order d = 0..D-1), two roundings to the input dtype, masks --------------------
+  float lmax = -INFINITY;
+  for (int j = tid; j < nk; j += 256) {
+    const uint4 *row = (const uint4 *)(pk_base + (size_t)j * D);
+    double acc = 0.0;
+#pragma unroll
+    for (int cch = 0; cch < D / 8; cch++) {
+      const uint4 v = row[cch];
+      const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+      for (int e = 0; e < 8; e++) {
+        const float kf = elem_to_f32<DT>((uint16_t)((e & 1) ? (w[e >> 1] >> 16) : (w[e >> 1] & 0xffffu)));
+        acc = acc + (double)s_pq[cch * 8 + e] * (double)kf;   // product exact in binary64
+      }
+    }
+    const float s1 = elem_to_f32<DT>(f64_to_elem<DT>(acc));
+    float s2 = elem_to_f32<DT>(f64_to_elem<DT>((double)s1 * (double)sm_scale));
+    if (!simk[j] || j >= causal_lim) s2 = -INFINITY;
+    s_score[j] = s2;
+    lmax = fmaxf(lmax, s2);
+  }
+  lmax = wave_max_f32(lmax);
+  if ((tid & 63) == 0) s_wmax[tid >> 6] = lmax;
+  __syncthreads();
+  const float mx = fmaxf(fmaxf(s_wmax[0], s_wmax[1]), fmaxf(s_wmax[2], s_wmax[3]));
+
+  // ---- exp and the fixed summation tree -------------------------------------------------------------
+  double part = 0.0;
+  for (int j = tid; j < nk; j += 256) {
+    const float s2 = s_score[j];
+    const double e = (s2 == -INFINITY) ? 0.0 : cexp((double)s2 - (double)mx);
+    e_buf[j] = e;
+    part = part + e;
+  }
+#pragma unroll
+  for (int o = 32; o >= 1; o >>= 1) part = part + shfl_xor_f64(part, o);
+  if ((tid & 63) == 0) s_wsum[tid >> 6] = part;
+  __syncthreads();
+  const double total = ((s_wsum[0] + s_wsum[1]) + s_wsum[2]) + s_wsum[3];
+
+  // ---- probabilities -> sortable keys (value bits, then lower index first) --------------------------
+  for (int j = tid; j < nk; j += 256) {
+    double p = e_buf[j] / total;
+    if (!__builtin_isfinite(p)) p = 0.0;
+    const uint32_t bits = f64_to_elem<DT>(p);
+    okey[j] = (bits << 16) | (0xffffu - (uint32_t)j);
+  }
+  __syncthreads();
+  for (int j = tid; j < nkp; j += 256) skey[j] = (j < nk) ? okey[j] : 0u;
+  __syncthreads();
+
+  // ---- bitonic sort, descending ----------------------------------------------------------------------
+  for (int k = 2; k <= nkp; k <<= 1) {
+    for (int j = k >> 1; j > 0; j >>= 1) {
+      for (int t = tid; t < nkp / 2; t += 256) {
+        const int lo = ((t / j) * 2 * j) + (t % j);
+        const int hi = lo + j;
+        const bool desc = (lo & k) == 0;
+        const uint32_t a = skey[lo], b = skey[hi];
+        if ((a < b) == desc) { skey[lo] = b; skey[hi] = a; }
+      }
+      __syncthreads();
+    }
+  }
+
+  // ---- how many to keep -------------------------------------------------------------------------------
+  long long n;
+  if (topk != nullptr) {
+    const float t = topk[h] * (float)nk;     // binary32 product, truncated (utils.py:405)
+    n = (long long)t;
+  } else {
+    // cdf[i] = T(sum_{u<=i} p_sorted[u]);  n = #{i < nk : cdf[i] <= threshold}  (utils.py:398-403)
+    const int seg = nkp / 256;
+    const int i0 = tid * seg;
+    double lsum = 0.0;
+    for (int u = 0; u < seg; u++) lsum += (double)elem_to_f32<DT>((uint16_t)(skey[i0 + u] >> 16));
+    s_tsum[tid] = lsum;
+    __syncthreads();
+    double run = 0.0;
+    for (int u = 0; u < tid; u++) run += s_tsum[u];
+    const double thr = (double)cdfthr[h];
+    int cnt = 0;
+    for (int u = 0; u < seg; u++) {
+      run += (double)elem_to_f32<DT>((uint16_t)(skey[i0 + u] >> 16));
+      const float cdfv = elem_to_f32<DT>(f64_to_elem<DT>(run));
+      if (i0 + u < nk && (double)cdfv <= thr) cnt++;
+    }
+    cnt = wave_sum_i32(cnt);
+    if (tid == 0) s_n = 0;
+    __syncthreads();
+    if ((tid & 63) == 0) atomicAdd(&s_n, cnt);
+    __syncthreads();
+    n = s_n;
+  }
+  if (n <= 0) n = 1;                              // utils.py:289
+  const uint32_t kth = (n >= nk) ? 0u : skey[n - 1];
+  __syncthreads();                                // skey is dead from here; s_idx may overwrite e_buf's upper half
+
+  // ---- block map row and LUT ---------------------------------------------------------------------------
+  const bool row_forced = sim_q[(size_t)bh * nq + i] == 0;
+  auto flag = [&](int j) -> bool {
+    bool f = row_forced || (okey[j] >= kth) || (simk[j] == 0);
+    if (j >= causal_lim) f = false;
+    if (sink && j == 0) f = true;
+    return f;
+  };
+  const size_t row_off = ((size_t)bh * nq + i) * nk;
+  if (bmap != nullptr)
+    for (int j = tid; j < nk; j += 256) bmap[row_off + j] = flag(j) ? 1 : 0;
+  emit_lut(flag, nk, nkp, s_idx, s_tmp, lut + row_off, valid + (size_t)bh * nq + i);
+}
+
+// =============================================================================================
+// user mask -> LUT
+// =============================================================================================
+template <int KIND>
+__device__ __forceinline__ bool mask_nonzero(const void *row, int j) {
+  if constexpr (KIND == 0) return ((const uint8_t *)row)[j] != 0;
+  if constexpr (KIND == 1) return ((const uint16_t *)row)[j] != 0;
+  if constexpr (KIND == 2) return ((const uint32_t *)row)[j] != 0;
+  if constexpr (KIND == 3) return ((const uint64_t *)row)[j] != 0;
+  if constexpr (KIND == 4) return (((const uint16_t *)row)[j] & 0x7fffu) != 0;            // +-0.0 is zero
+  if constexpr (KIND == 5) return (((const uint32_t *)row)[j] & 0x7fffffffu) != 0;
+  if constexpr (KIND == 6) return (((const uint64_t *)row)[j] & 0x7fffffffffffffffull) != 0;
+  return false;
+}
+constexpr int mask_elem_size(int kind) { return kind == 0 ? 1 : (kind == 1 || kind == 4) ? 2 : (kind == 2 || kind == 5) ? 4 : 8; }
+
+template <int KIND>
+__global__ __launch_bounds__(256) void map_to_lut_kernel(const void *__restrict__ mask, int32_t *__restrict__ lut,
+                                                         int32_t *__restrict__ valid, int nq, int nk, int nkp) {
+  extern __shared__ __align__(16) unsigned char smem[];
+  int32_t *s_idx = (int32_t *)smem;
+  __shared__ int s_tmp[256];
+  const int i = blockIdx.x, bh = blockIdx.y;
+  const size_t row_off = ((size_t)bh * nq + i) * nk;
+  const void *row = (const unsigned char *)mask + row_off * mask_elem_size(KIND);
+  auto flag = [&](int j) -> bool { return mask_nonzero<KIND>(row, j); };
+  emit_lut(flag, nk, nkp, s_idx, s_tmp, lut + row_off, valid + (size_t)bh * nq + i);
+}
+
+// =============================================================================================
+// host launchers
+// =============================================================================================
+static int next_pow2_ge(int v, int lo) {
+  int p = lo;
+  while (p < v) p <<= 1;
+  return p;
+}
+
+static int km_chunks(int B, int H, int N) {
+  // enough workgroups to fill 256 CUs several times over, at least 256 rows each
+  int want = (4096 + B * H - 1) / (B * H);
+  int maxc = (N + 255) / 256;
+  int c = want < maxc ? want : maxc;
+  return c < 1 ? 1 : c;
+}
+
+size_t km_mean_workspace_bytes(int B, int H, int N, int D) {
+  return (size_t)B * H * km_chunks(B, H, N) * D * sizeof(double);
+}
+
+template <int D, int DT>
+static void launch_km(const void *k, void *km, void *ws, int B, int H, int N, hipStream_t st) {
+  const int nchunk = km_chunks(B, H, N);
+  const int rpc = (N + nchunk - 1) / nchunk;
+  km_partial_kernel<D, DT><<<dim3(nchunk, B * H), 256, 0, st>>>((const uint16_t *)k, (double *)ws, N, rpc);
+  km_final_kernel<DT><<<B * H, D, 0, st>>>((const double *)ws, (uint16_t *)km, nchunk, D, N);
+}
+
+void launch_km_mean(const void *k, void *km, void *ws, int B, int H, int N, int D, int dtype, hipStream_t st) {
+  if (D == 64) { if (dtype == 0) launch_km<64, 0>(k, km, ws, B, H, N, st); else launch_km<64, 1>(k, km, ws, B, H, N, st); }
+  else         { if (dtype == 0) launch_km<128, 0>(k, km, ws, B, H, N, st); else launch_km<128, 1>(k, km, ws, B, H, N, st); }
+}
+
+template <int BS, int D, int DT>
+static void launch_psq3(const void *x, const void *km, void *pool, uint8_t *sim, int8_t *xq, float *scale,
+                        const float *thr, int B, int H, int N, hipStream_t st) {
+  const int nb = (N + BS - 1) / BS;
+  const dim3 grid(nb, B * H);
+  const uint16_t *xp = (const uint16_t *)x, *kp = (const uint16_t *)km;
+  uint16_t *pp = (uint16_t *)pool;
+  if (pool != nullptr) {
+    if (km) pool_sim_quant_kernel<BS, D, DT, true, true><<<grid, 256, 0, st>>>(xp, kp, pp, sim, xq, scale, thr, H, N, nb);
+    else    pool_sim_quant_kernel<BS, D, DT, false, true><<<grid, 256, 0, st>>>(xp, kp, pp, sim, xq, scale, thr, H, N, nb);
+  } else {
+    if (km) pool_sim_quant_kernel<BS, D, DT, true, false><<<grid, 256, 0, st>>>(xp, kp, pp, sim, xq, scale, thr, H, N, nb);
+    else    pool_sim_quant_kernel<BS, D, DT, false, false><<<grid, 256, 0, st>>>(xp, kp, pp, sim, xq, scale, thr, H, N, nb);
+  }
+}
+
+void launch_pool_sim_quant(const void *x, const void *km, void *pool, uint8_t *sim, int8_t *xq, float *scale,
+                           const float *thr, int B, int H, int N, int D, int block, int dtype, hipStream_t st) {
+#define SPG_PSQ(BS_, D_, DT_) launch_psq3<BS_, D_, DT_>(x, km, pool, sim, xq, scale, thr, B, H, N, st)
+  if (block == 128) {
+    if (D == 64) { if (dtype == 0) SPG_PSQ(128, 64, 0); else SPG_PSQ(128, 64, 1); }
+    else         { if (dtype == 0) SPG_PSQ(128, 128, 0); else SPG_PSQ(128, 128, 1); }
+  } else {
+    if (D == 64) { if (dtype == 0) SPG_PSQ(64, 64, 0); else SPG_PSQ(64, 64, 1); }
+    else         { if (dtype == 0) SPG_PSQ(64, 128, 0); else SPG_PSQ(64, 128, 1); }
+  }
+#undef SPG_PSQ
+}
+
+int block_select_max_nk() { return 8192; }
+
+template <int D, int DT>
+static hipError_t launch_bs2(const void *pq, const uint8_t *sq, const void *pk, const uint8_t *sk, const float *topk,
+                             const float *cdf, int causal, int sink, int32_t *lut, int32_t *valid, uint8_t *bmap, int B,
+                             int H, int nq, int nk, hipStream_t st) {
+  const int nkp = next_pow2_ge(nk, 256);
+  const size_t lds = 12 * (size_t)nkp;
+  auto kern = block_select_kernel<D, DT>;
+  if (lds > 48 * 1024) {
+    hipError_t e = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    if (e != hipSuccess) return e;
+  }
+  kern<<<dim3(nq, B * H), 256, lds, st>>>((const uint16_t *)pq, sq, (const uint16_t *)pk, sk, topk, cdf, causal, sink, lut,
+                                         valid, bmap, H, nq, nk, nkp);
+  return hipSuccess;
+}
+
+hipError_t launch_block_select(const void *pq, const uint8_t *sq, const void *pk, const uint8_t *sk, const float *topk,
+                               const float *cdf, int causal, int sink, int32_t *lut, int32_t *valid, uint8_t *bmap,
+                               int B, int H, int nq, int nk, int D, int dtype, hipStream_t st) {
+#define SPG_BS(D_, DT_) return launch_bs2<D_, DT_>(pq, sq, pk, sk, topk, cdf, causal, sink, lut, valid, bmap, B, H, nq, nk, st)
+  if (D == 64) { if (dtype == 0) SPG_BS(64, 0); else SPG_BS(64, 1); }
+  else         { if (dtype == 0) SPG_BS(128, 0); else SPG_BS(128, 1); }
+#undef SPG_BS
+}
+
+hipError_t launch_map_to_lut(const void *mask, int kind, int32_t *lut, int32_t *valid, int B, int H, int nq, int nk,
+                             hipStream_t st) {
+  const int nkp = next_pow2_ge(nk, 256);
+  const size_t lds = 4 * (size_t)nkp;
+  const dim3 grid(nq, B * H);
+#define SPG_M2L(K_)                                                                                      \
+  case K_: {                                                                                             \
+    auto kern = map_to_lut_kernel<K_>;                                                                   \
+    if (lds > 48 * 1024) {                                                                               \
+      hipError_t e = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds); \
+      if (e != hipSuccess) return e;                                                                     \
+    }                                                                                                    \
+    kern<<<grid, 256, lds, st>>>(mask, lut, valid, nq, nk, nkp);                                         \
+    break;                                                                                               \
+  }
+  switch (kind) {
+    SPG_M2L(0) SPG_M2L(1) SPG_M2L(2) SPG_M2L(3) SPG_M2L(4) SPG_M2L(5) SPG_M2L(6)
+    default: return hipErrorInvalidValue;
+  }
+#undef SPG_M2L
+  return hipSuccess;
+}
+
+}  // namespace spg

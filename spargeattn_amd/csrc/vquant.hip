@@ -1,0 +1,129 @@
+// V path for gfx950: fp16 cast, per-(b,h,channel) absmax, FP8 e4m3 quantisation written straight into the
+// [B][H][nk][D][64] tile layout the attention kernel's V^T operand reads.
+// Replaces TransposePadPermuteKernel + MeanScaleKernel (csrc/fused/fused.cu:26-77, 80-191) called with
+// scale_max = 2.25 (spas_sage_attn/core.py:147-151).  HBM-bound: V is read twice (absmax, quantise), written once
+// at 1 B/element.  Compile with -ffp-contract=off.
+#include "common.h"
+#include "launch.h"
+
+namespace spg {
+
+template <int DT>
+__device__ __forceinline__ float elem_to_f16_f32(uint16_t b) {
+  // value of the element after the cast to fp16 the reference applies to V (core.py:117)
+  if constexpr (DT == 0) return elem_to_f32<0>(b);
+  const _Float16 h = (_Float16)elem_to_f32<1>(b);
+  return (float)h;
+}
+
+__global__ void fill_u32_kernel(uint32_t *p, uint32_t v, int n) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) p[i] = v;
+}
+
+template <int D, int DT>
+__global__ __launch_bounds__(256) void v_absmax_kernel(const uint16_t *__restrict__ v, uint32_t *__restrict__ amax_bits,
+                                                       int N, int rows_per_chunk) {
+  constexpr int TPR = D / 8;
+  constexpr int RPP = 256 / TPR;
+  const int bh = blockIdx.y, chunk = blockIdx.x;
+  const int c = threadIdx.x % TPR, r = threadIdx.x / TPR;
+  const int row0 = chunk * rows_per_chunk;
+  const int row1 = min(N, row0 + rows_per_chunk);
+  const uint16_t *base = v + (size_t)bh * N * D + c * 8;
+  float m[8];
+#pragma unroll
+  for (int e = 0; e < 8; e++) m[e] = 0.f;
+#pragma unroll 4
+  for (int row = row0 + r; row < row1; row += RPP) {
+    const uint4 q = *(const uint4 *)(base + (size_t)row * D);
+    const uint32_t w[4] = {q.x, q.y, q.z, q.w};
+#pragma unroll
+    for (int e = 0; e < 8; e++) {
+      const uint16_t b = (uint16_t)((e & 1) ? (w[e >> 1] >> 16) : (w[e >> 1] & 0xffffu));
+      m[e] = fmaxf(m[e], fabsf(elem_to_f16_f32<DT>(b)));
+    }
+  }
+  __shared__ float sm[RPP][D];
+#pragma unroll
+  for (int e = 0; e < 8; e++) sm[r][c * 8 + e] = m[e];
+  __syncthreads();
+  if (threadIdx.x < D) {
+    float s = 0.f;
+    for (int i = 0; i < RPP; i++) s = fmaxf(s, sm[i][threadIdx.x]);
+    // non-negative floats order like their bit patterns; max is order independent
+    atomicMax(amax_bits + (size_t)bh * D + threadIdx.x, __builtin_bit_cast(uint32_t, s));
+  }
+}
+
+// One workgroup per 64-key tile.  LDS holds the transposed tile [D][64] bytes.
+template <int D, int DT>
+__global__ __launch_bounds__(256) void v_quant_kernel(const uint16_t *__restrict__ v, const float *__restrict__ amax,
+                                                      uint8_t *__restrict__ v8, int N, int nk) {
+  constexpr int TPR = D / 8;
+  constexpr int RPP = 256 / TPR;
+  constexpr int NP = 64 / RPP;
+  constexpr int LDW = 64 + 4;  // padded row (bytes) of the transposed tile
+  __shared__ __align__(16) uint8_t tile[D * LDW];
+  const int blk = blockIdx.x, bh = blockIdx.y, tid = threadIdx.x;
+  const int c = tid % TPR, r = tid / TPR;
+  float recp[8];
+#pragma unroll
+  for (int e = 0; e < 8; e++) recp[e] = 2.25f / amax[(size_t)bh * D + c * 8 + e];
+  const uint16_t *base = v + ((size_t)bh * N + (size_t)blk * 64) * D + c * 8;
+#pragma unroll
+  for (int p = 0; p < NP; p++) {
+    const int row = r + p * RPP;
+    const bool ok = blk * 64 + row < N;
+    uint4 q = make_uint4(0, 0, 0, 0);
+    if (ok) q = *(const uint4 *)(base + (size_t)row * D);
+    const uint32_t w[4] = {q.x, q.y, q.z, q.w};
+#pragma unroll
+    for (int e = 0; e < 8; e += 2) {
+      const float a = elem_to_f16_f32<DT>((uint16_t)(w[e >> 1] & 0xffffu)) * recp[e];
+      const float b = elem_to_f16_f32<DT>((uint16_t)(w[e >> 1] >> 16)) * recp[e + 1];
+      const int pk = ok ? __builtin_amdgcn_cvt_pk_fp8_f32(a, b, 0, false) : 0;   // rows beyond N are zero
+      tile[(c * 8 + e) * LDW + row] = (uint8_t)(pk & 0xff);
+      tile[(c * 8 + e + 1) * LDW + row] = (uint8_t)((pk >> 8) & 0xff);
+    }
+  }
+  __syncthreads();
+  uint8_t *out = v8 + ((size_t)bh * nk + blk) * (size_t)(D * 64);
+  for (int i = tid; i < D * 4; i += 256) {   // 16-byte pieces: D rows x 4
+    const int d = i >> 2, part = i & 3;
+    const uint32_t *src = (const uint32_t *)(tile + d * LDW + part * 16);
+    *(uint4 *)(out + d * 64 + part * 16) = make_uint4(src[0], src[1], src[2], src[3]);
+  }
+}
+
+__global__ void v_scale_final_kernel(float *v_scale, int n) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) v_scale[i] = v_scale[i] / 2.25f;
+}
+
+static int v_chunks(int B, int H, int N) {
+  int want = (4096 + B * H - 1) / (B * H);
+  int maxc = (N + 255) / 256;
+  int c = want < maxc ? want : maxc;
+  return c < 1 ? 1 : c;
+}
+
+template <int D, int DT>
+static void launch_vq2(const void *v, uint8_t *v8, float *v_scale, int B, int H, int N, hipStream_t st) {
+  const int n = B * H * D;
+  const int nk = (N + 63) / 64;
+  const int nchunk = v_chunks(B, H, N);
+  const int rpc = (N + nchunk - 1) / nchunk;
+  fill_u32_kernel<<<(n + 255) / 256, 256, 0, st>>>((uint32_t *)v_scale, 0u, n);
+  v_absmax_kernel<D, DT><<<dim3(nchunk, B * H), 256, 0, st>>>((const uint16_t *)v, (uint32_t *)v_scale, N, rpc);
+  v_quant_kernel<D, DT><<<dim3(nk, B * H), 256, 0, st>>>((const uint16_t *)v, v_scale, v8, N, nk);
+  v_scale_final_kernel<<<(n + 255) / 256, 256, 0, st>>>(v_scale, n);
+}
+
+void launch_v_quant_fp8(const void *v, uint8_t *v8, float *v_scale, int B, int H, int N, int D, int dtype,
+                        hipStream_t st) {
+  if (D == 64) { if (dtype == 0) launch_vq2<64, 0>(v, v8, v_scale, B, H, N, st); else launch_vq2<64, 1>(v, v8, v_scale, B, H, N, st); }
+  else         { if (dtype == 0) launch_vq2<128, 0>(v, v8, v_scale, B, H, N, st); else launch_vq2<128, 1>(v, v8, v_scale, B, H, N, st); }
+}
+
+}  // namespace spg

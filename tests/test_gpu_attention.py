@@ -1,0 +1,189 @@
+"""GPU parity of the block-sparse attention kernel and of the operator API against the oracle.
+
+Tolerances (floating point, approximate exp2/rcp on both sides): cosine similarity >= 0.999 and
+relative L1 <= 1e-2 against the oracle; the quantised tensors, scales, block maps and LUTs are bit-exact.
+"""
+import numpy as np
+import pytest
+import torch
+
+import spargeattn_amd as sa
+from oracle import api as oapi, attention as oat, maskpred as mp
+from spargeattn_amd import _lib, utils, workloads as W
+from gpu_common import tag_of, to_np, bits_equal_T, v8_natural, rand_T
+
+pytestmark = pytest.mark.gpu
+
+COS_MIN, L1_MAX = 0.999, 1e-2
+
+
+def _check_out(o_gpu, ref_out, written=None):
+    got = to_np(o_gpu)
+    if written is not None:
+        rows = np.repeat(written, 128, axis=2)[:, :, :got.shape[2]]
+        got, ref_out = got[rows], ref_out[rows]
+    if not np.any(ref_out):                      # degenerate case (everything skipped): exact zeros on both sides
+        assert not np.any(got)
+        return None
+    met = oat.precision_metric(got, ref_out)
+    assert met["Cossim"] >= COS_MIN and met["L1"] <= L1_MAX, met
+    return met
+
+
+def _stage_inputs(B, H, N, D, dtype, seed):
+    q = rand_T((B, H, N, D), dtype, seed)
+    k = rand_T((B, H, N, D), dtype, seed + 1, shift=0.4)
+    v = rand_T((B, H, N, D), dtype, seed + 2)
+    return q, k, v
+
+
+def _run_kernel_on_oracle_tensors(res, out_dtype, H, N, D, pvthreshd, is_causal=False):
+    """Feeds the ORACLE's quantised tensors to the HIP attention kernel (isolates the kernel)."""
+    dev = "cuda"
+    q8 = torch.from_numpy(res["q8"]).to(dev)
+    k8 = torch.from_numpy(res["k8"]).to(dev)
+    B = q8.shape[0]
+    nk = (N + 63) // 64
+    v8_nat = torch.from_numpy(res["v8"][:, :, :nk * 64]).to(dev)            # (B,H,nk*64,D)
+    v8 = v8_nat.view(B, H, nk, 64, D).permute(0, 1, 2, 4, 3).contiguous()  # tile layout
+    out = torch.zeros((B, H, N, D), dtype=out_dtype, device=dev)
+    pvt = torch.full((H,), float(pvthreshd), dtype=torch.float32, device=dev)
+    pvc = _lib.block_sparse_attn(q8, k8, v8, out, torch.from_numpy(res["lut"]).to(dev),
+                                 torch.from_numpy(res["valid"]).to(dev), pvt,
+                                 torch.from_numpy(res["q_scale"]).to(dev), torch.from_numpy(res["k_scale"]).to(dev),
+                                 torch.from_numpy(res["v_scale"]).to(dev), 1.0 / D ** 0.5, is_causal=is_causal,
+                                 return_pv_count=True)
+    torch.cuda.synchronize()
+    return out, pvc
+
+
+@pytest.mark.parametrize("dtype,D,N", [(torch.bfloat16, 128, 1024), (torch.float16, 64, 1024),
+                                       (torch.bfloat16, 64, 333), (torch.float16, 128, 700)])
+@pytest.mark.parametrize("topk", [0.5, 1.0])
+def test_attention_kernel_on_oracle_tensors(dtype, D, N, topk):
+    B, H = 1, 2
+    q, k, v = _stage_inputs(B, H, N, D, dtype, 30)
+    res = oapi.spas_sage2_attn_meansim_topk(to_np(q), to_np(k), to_np(v), tag_of(dtype), topk=topk)
+    out, pvc = _run_kernel_on_oracle_tensors(res, dtype, H, N, D, 50)
+    _check_out(out, res["out"])
+    assert np.array_equal(pvc.cpu().numpy(), res["pv_count"])
+    assert np.array_equal(res["pv_count"], res["valid"])
+
+
+@pytest.mark.parametrize("kernel_causal", [False, True])
+def test_attention_kernel_causal(kernel_causal):
+    dtype, D, N, B, H = torch.bfloat16, 128, 1024, 1, 2
+    q, k, v = _stage_inputs(B, H, N, D, dtype, 40)
+    res = oapi.spas_sage2_attn_meansim_topk(to_np(q), to_np(k), to_np(v), tag_of(dtype), topk=0.6, is_causal=True,
+                                            kernel_causal=kernel_causal)
+    out, _ = _run_kernel_on_oracle_tensors(res, dtype, H, N, D, 50, is_causal=kernel_causal)
+    _check_out(out, res["out"])
+
+
+def test_attention_kernel_pv_threshold_and_empty_rows():
+    dtype, D, N, B, H = torch.float16, 64, 768, 1, 2
+    q = (rand_T((B, H, N, D), dtype, 50).float().abs() + 0.5).to(dtype)
+    k = rand_T((B, H, N, D), dtype, 51, scale=0.05)
+    k[:, :, :64] += 6.0                                     # block 0 dominates: later blocks fall below the threshold
+    v = rand_T((B, H, N, D), dtype, 52)
+    mask = np.ones((B, H, 6, 12), np.int32)
+    mask[0, 1, 2] = 0                                       # a row block without any K block
+    for thr in (1e6, 5.0, -1e6, -1e7):
+        res = oapi.block_sparse_sage2_attn(to_np(q), to_np(k), to_np(v), mask, tag_of(dtype), pvthreshd=thr)
+        out, pvc = _run_kernel_on_oracle_tensors(res, dtype, H, N, D, thr)
+        assert np.array_equal(pvc.cpu().numpy(), res["pv_count"]), thr
+        _check_out(out, res["out"], written=res["written"])
+        assert torch.all(out[0, 1, 256:384] == 0)           # untouched (buffer was zero-initialised by the test)
+    assert res["pv_count"].max() == 2 and res["pv_count"][0, 1, 2] == 0
+
+
+@pytest.mark.parametrize("name,shrink", [("cfg1", None), ("cfg3", dict(H=2, grid=(4, 12, 15), text_tokens=50)),
+                                         ("cfg4", dict(H=2, N=2048)), ("cfg5", dict(H=2, grid=(3, 10, 22)))])
+def test_topk_api_end_to_end(name, shrink):
+    cfg = W.CONFIGS[name]
+    q, k, v = W.make_qkv(cfg, device="cpu", shrink=shrink)
+    tag = tag_of(cfg.dtype)
+    res = oapi.spas_sage2_attn_meansim_topk(to_np(q), to_np(k), to_np(v), tag, is_causal=cfg.is_causal,
+                                            topk=cfg.topk, pvthreshd=cfg.pvthreshd)
+    qg, kg, vg = q.cuda(), k.cuda(), v.cuda()
+    # stage by stage through the host API (bit-exact)
+    km = _lib.km_mean(kg)
+    assert bits_equal_T(km[:, :, 0], res["km"], cfg.dtype)
+    bmap, q8, qs, k8, ks = utils.get_block_map_meansim_fuse_quant(qg, kg, km, is_causal=cfg.is_causal,
+                                                                  simthreshd1=-0.1, cdfthreshd=None, topk=cfg.topk)
+    assert np.array_equal(q8.cpu().numpy(), res["q8"]) and np.array_equal(k8.cpu().numpy(), res["k8"])
+    assert np.array_equal(qs.cpu().numpy(), res["q_scale"]) and np.array_equal(ks.cpu().numpy(), res["k_scale"])
+    assert np.array_equal(bmap.cpu().numpy(), res["map"])
+    lut, valid, *_ = utils.get_block_map_meansim_fuse_quant(qg, kg, km, is_causal=cfg.is_causal, simthreshd1=-0.1,
+                                                            cdfthreshd=None, topk=cfg.topk, return_lut=True)
+    assert np.array_equal(lut.cpu().numpy(), res["lut"]) and np.array_equal(valid.cpu().numpy(), res["valid"])
+    v8, vs = _lib.v_quant_fp8(vg.to(torch.float16))
+    N = q.shape[2]
+    assert np.array_equal(v8_natural(v8, N), res["v8"][:, :, :N]) and np.array_equal(vs.cpu().numpy(), res["v_scale"])
+    # the operator itself
+    o, sparsity = sa.spas_sage2_attn_meansim_topk_cuda(qg, kg, vg, is_causal=cfg.is_causal, topk=cfg.topk,
+                                                       pvthreshd=cfg.pvthreshd, return_sparsity=True)
+    assert o.dtype == cfg.dtype and o.shape == q.shape
+    assert abs(sparsity - res["sparsity"]) < 1e-6
+    _check_out(o, res["out"])
+    # NHD layout gives the same numbers
+    o2 = sa.spas_sage2_attn_meansim_topk_cuda(qg.transpose(1, 2).contiguous(), kg.transpose(1, 2).contiguous(),
+                                              vg.transpose(1, 2).contiguous(), is_causal=cfg.is_causal, topk=cfg.topk,
+                                              pvthreshd=cfg.pvthreshd, tensor_layout="NHD")
+    assert torch.equal(o2.transpose(1, 2), o)
+
+
+def test_mask_api_end_to_end_cfg2_shape():
+    cfg = W.CONFIGS["cfg2"]
+    B, H, N = 1, 3, 1024
+    q, k, v = W.make_qkv(cfg, device="cpu", shrink=dict(B=B, H=H, N=N))
+    mask = W.make_mask_id(cfg, B, H, N)
+    res = oapi.block_sparse_sage2_attn(to_np(q), to_np(k), to_np(v), mask.numpy(), tag_of(cfg.dtype))
+    o, sparsity = sa.block_sparse_sage2_attn_cuda(q.cuda(), k.cuda(), v.cuda(), mask_id=mask.cuda(),
+                                                  return_sparsity=True)
+    assert abs(sparsity - res["sparsity"]) < 1e-6
+    _check_out(o, res["out"])
+    # masked fp32 reference (what config 2 is specified against): error of the method, reported
+    tm = utils.block_map_to_mask(mask.bool())[:, :, :N, :N].cuda()
+    ref = torch.nn.functional.scaled_dot_product_attention(q.cuda().float(), k.cuda().float(), v.cuda().float(),
+                                                           attn_mask=tm)
+    met = oat.precision_metric(to_np(o), to_np(ref))
+    assert met["Cossim"] > 0.995, met
+
+
+def test_cdf_api_end_to_end():
+    dtype, D, N, B, H = torch.bfloat16, 64, 1024, 1, 2
+    q, k, v = W.make_qkv(W.CONFIGS["cfg1"], device="cpu")
+    q, k, v = q.to(dtype), k.to(dtype), v.to(dtype)
+    res = oapi.spas_sage2_attn_meansim_topk(to_np(q), to_np(k), to_np(v), tag_of(dtype), simthreshd1=0.6,
+                                            cdfthreshd=0.98, topk=None, attention_sink=True)
+    o, sp = sa.spas_sage2_attn_meansim_cuda(q.cuda(), k.cuda(), v.cuda(), attention_sink=True, return_sparsity=True)
+    assert abs(sp - res["sparsity"]) < 1e-6
+    _check_out(o, res["out"])
+
+
+def test_fp32_input_and_error_paths():
+    q = torch.randn(1, 2, 256, 64, device="cuda")
+    o = sa.spas_sage2_attn_meansim_topk_cuda(q, q, q)
+    assert o.dtype == torch.float16
+    with pytest.raises(NameError):
+        sa.spas_sage2_attn_meansim_topk_cuda(q, q, q, smooth_k=False)
+    with pytest.raises(AssertionError, match="headdim"):
+        q96 = torch.randn(1, 2, 256, 96, device="cuda", dtype=torch.float16)
+        sa.spas_sage2_attn_meansim_topk_cuda(q96, q96, q96)
+    with pytest.raises(AssertionError, match="Only one of cdfthreshd and topk"):
+        sa.spas_sage2_attn_meansim_topk_cuda(q, q, q, cdfthreshd=0.9, topk=0.5)
+    with pytest.raises(ValueError):
+        sa.spas_sage2_attn_meansim_topk_cuda(q, q, q, topk="half")
+    o = sa.spas_sage2_attn_meansim_topk_cuda(q, q, q, topk=torch.tensor([0.5, 0.25], device="cuda"))
+    assert torch.isfinite(o.float()).all()
+
+
+@pytest.mark.parametrize("D,N,causal", [(128, 1024, False), (128, 1024, True), (64, 700, False), (64, 512, True)])
+def test_dense_f16_comparator(D, N, causal):
+    B, H = 1, 2
+    q, k, v = (rand_T((B, H, N, D), torch.float16, 60 + i) for i in range(3))
+    o = _lib.dense_attn_f16(q, k, _lib.v_tiles_f16(v), 1.0 / D ** 0.5, is_causal=causal)
+    ref = torch.nn.functional.scaled_dot_product_attention(q.float(), k.float(), v.float(), is_causal=causal)
+    met = oat.precision_metric(to_np(o), to_np(ref))
+    assert met["Cossim"] > 0.9999 and met["L1"] < 5e-3, met

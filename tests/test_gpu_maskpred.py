@@ -1,0 +1,127 @@
+"""GPU parity (bit-exact) of the mask-prediction / quantisation kernels against the oracle, through the C ABI."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import maskpred as mp
+from oracle import vquant as vq
+from spargeattn_amd import _lib
+from gpu_common import tag_of, to_np, bits_equal_T, v8_natural, rand_T
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("B,H,N,D", [(1, 2, 1024, 64), (2, 3, 333, 128), (1, 1, 5000, 128)])
+def test_km_mean(dtype, B, H, N, D):
+    k = rand_T((B, H, N, D), dtype, 1, shift=0.3)
+    km = _lib.km_mean(k)
+    assert km.shape == (B, H, 1, D) and km.dtype == dtype
+    assert bits_equal_T(km[:, :, 0], mp.km_mean(to_np(k), tag_of(dtype)), dtype)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("B,H,N,D", [(1, 2, 1024, 64), (2, 2, 333, 128), (1, 3, 1100, 128), (1, 2, 200, 64)])
+def test_pool_sim_quant(dtype, B, H, N, D):
+    tag = tag_of(dtype)
+    q = rand_T((B, H, N, D), dtype, 2)
+    k = rand_T((B, H, N, D), dtype, 3, shift=0.5)
+    # second head: strongly self-similar rows so that both sim outcomes occur with threshold 0.5
+    base = rand_T((B, 1, 1, D), dtype, 4)
+    k[:, 1:2] = (base.float() * 4 + k[:, 1:2].float() * 0.3).to(dtype)
+    q[:, 1:2] = (base.float() * 4 + q[:, 1:2].float() * 0.3).to(dtype)
+    thr = torch.tensor([0.5] * H, dtype=torch.float32, device="cuda")
+    km = _lib.km_mean(k)
+    for x, mean, bs in ((q, None, 128), (k, km, 64)):
+        pool, sim, xq, scale = _lib.pool_sim_quant(x, mean, bs, thr)
+        ref = mp.pool_sim_quant(to_np(x), None if mean is None else to_np(mean[:, :, 0]), bs, thr.cpu().numpy(), tag)
+        assert np.array_equal(xq.cpu().numpy(), ref["q"])
+        assert np.array_equal(scale.cpu().numpy().view(np.uint32), ref["scale"].view(np.uint32))
+        assert bits_equal_T(pool, ref["pool"], dtype)
+        assert np.array_equal(sim.cpu().numpy(), ref["sim"])
+        if mean is None:      # (K loses the shared component when km is subtracted)
+            assert ref["sim"][:, 1, 0].all() and not ref["sim"][:, 0, 0].any()   # both outcomes are exercised
+        if N % bs:
+            assert not ref["sim"][:, :, -1].any()                                # partial block is never "similar"
+        # quant-only entry (A13) gives the same integers and scales
+        _, _, xq2, scale2 = _lib.pool_sim_quant(x, mean, bs, with_pool=False)
+        assert torch.equal(xq2, xq) and torch.equal(scale2, scale)
+
+
+def _pools(B, H, nq, nk, D, dtype, seed):
+    pq = rand_T((B, H, nq, D), dtype, seed, scale=1.5)
+    pk = rand_T((B, H, nk, D), dtype, seed + 1, scale=1.5)
+    g = torch.Generator().manual_seed(seed + 2)
+    sq = (torch.rand((B, H, nq), generator=g) > 0.15).cuda()
+    sk = (torch.rand((B, H, nk), generator=g) > 0.1).cuda()
+    return pq, sq, pk, sk
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("nq,nk,D", [(8, 16, 64), (5, 9, 128), (139, 278, 64), (40, 300, 128), (3, 700, 128)])
+@pytest.mark.parametrize("mode", ["topk", "topk_causal", "cdf", "cdf_causal_sink"])
+def test_block_select(dtype, nq, nk, D, mode):
+    tag = tag_of(dtype)
+    B, H = 1, 3
+    pq, sq, pk, sk = _pools(B, H, nq, nk, D, dtype, 10 + nq)
+    causal = "causal" in mode and nk == 2 * nq
+    sink = "sink" in mode
+    topk = cdf = None
+    if mode.startswith("topk"):
+        topk = torch.tensor([0.5, 0.3, 0.001], dtype=torch.float32, device="cuda")
+    else:
+        cdf = torch.tensor([0.9, 0.5, 0.999], dtype=torch.float32, device="cuda")
+    lut, valid, bmap = _lib.block_select(pq, sq, pk, sk, topk=topk, cdfthreshd=cdf, is_causal=causal,
+                                         attention_sink=sink, return_map=True)
+    ref_map = mp.block_map(to_np(pq), sq.cpu().numpy(), to_np(pk), sk.cpu().numpy(), tag, is_causal=causal,
+                           topk=None if topk is None else topk.cpu().numpy(),
+                           cdfthreshd=None if cdf is None else cdf.cpu().numpy(), attention_sink=sink)
+    ref_lut, ref_valid = mp.map_to_lut(ref_map)
+    got_map = bmap.cpu().numpy()
+    assert np.array_equal(got_map, ref_map), f"{(got_map != ref_map).sum()} of {ref_map.size} map entries differ"
+    assert np.array_equal(valid.cpu().numpy(), ref_valid)
+    assert np.array_equal(lut.cpu().numpy(), ref_lut)
+
+
+def test_block_select_rejects_bad_arguments():
+    pq, sq, pk, sk = _pools(1, 1, 4, 8, 64, torch.float16, 5)
+    t = torch.tensor([0.5], device="cuda")
+    with pytest.raises(ValueError, match="Only one of cdfthreshd and topk"):
+        _lib.block_select(pq, sq, pk, sk, topk=t, cdfthreshd=t)
+    with pytest.raises(ValueError, match="Only one of cdfthreshd and topk"):
+        _lib.block_select(pq, sq, pk, sk)
+
+
+@pytest.mark.parametrize("mdtype", [torch.bool, torch.uint8, torch.int32, torch.int64, torch.float16, torch.bfloat16,
+                                    torch.float32])
+def test_map_to_lut(mdtype):
+    g = torch.Generator().manual_seed(7)
+    m = torch.rand((2, 3, 11, 301), generator=g) < 0.3
+    m[0, 0, 0] = False
+    m[0, 0, 1] = True
+    mm = m.to(mdtype).cuda()
+    if mdtype.is_floating_point:
+        mm = mm * -2.5 if mdtype != torch.bool else mm
+    lut, valid = _lib.map_to_lut(mm.contiguous())
+    ref_lut, ref_valid = mp.map_to_lut(m.numpy())
+    assert np.array_equal(lut.cpu().numpy(), ref_lut) and np.array_equal(valid.cpu().numpy(), ref_valid)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("B,H,N,D", [(1, 2, 1024, 64), (2, 2, 333, 128), (1, 1, 4100, 128)])
+def test_v_quant_fp8(dtype, B, H, N, D):
+    v = rand_T((B, H, N, D), dtype, 20)
+    v[:, :, :, 1] *= 0.01
+    v8, v_scale = _lib.v_quant_fp8(v)
+    ref_codes, ref_scale = vq.v_quant_fp8(vq.to_fp16(to_np(v)))
+    nk = (N + 63) // 64
+    assert v8.shape == (B, H, nk, D, 64)
+    nat = v8_natural(v8)
+    assert np.array_equal(nat[:, :, :N], ref_codes[:, :, :N])
+    assert np.all(nat[:, :, N:] == 0)
+    assert np.array_equal(v_scale.cpu().numpy().view(np.uint32), ref_scale.view(np.uint32))
+    # hardware e4m3 convert agrees with torch's float8_e4m3fn cast on the same products
+    v16 = v.to(torch.float16).float()
+    recp = torch.from_numpy(np.float32(2.25) / v16.abs().amax(dim=2).cpu().numpy()).cuda()
+    lib = (v16 * recp[:, :, None, :]).to(torch.float8_e4m3fn).view(torch.uint8).cpu().numpy()
+    assert np.array_equal(nat[:, :, :N], lib)

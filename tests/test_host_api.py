@@ -1,0 +1,57 @@
+"""Host logic that needs no GPU: hyper-parameter handling, error behaviour, workload generators."""
+import pytest
+import torch
+
+from spargeattn_amd import utils, workloads as W
+import spargeattn_amd as sa
+
+
+def test_hyperparameter_check():
+    t = utils.hyperparameter_check(0.5, 4, "cpu")
+    assert t.shape == (4,) and t.dtype == torch.float32 and torch.all(t == 0.5)
+    assert torch.all(utils.hyperparameter_check(3, 2, "cpu") == 3.0)
+    assert torch.all(utils.hyperparameter_check(torch.tensor(0.25), 3, "cpu") == 0.25)
+    v = torch.tensor([0.1, 0.2, 0.3])
+    assert torch.equal(utils.hyperparameter_check(v, 3, "cpu"), v)
+    with pytest.raises(AssertionError):
+        utils.hyperparameter_check(v, 4, "cpu")
+    with pytest.raises(AssertionError):
+        utils.hyperparameter_check(torch.zeros(2, 2), 4, "cpu")
+    with pytest.raises(ValueError):
+        utils.hyperparameter_check("0.5", 4, "cpu")
+
+
+def test_api_preconditions_raise_like_the_reference():
+    q = torch.zeros(1, 2, 64, 64, dtype=torch.float16)
+    with pytest.raises(AssertionError, match="seq_len"):
+        sa.spas_sage2_attn_meansim_topk_cuda(q, q, q)
+    with pytest.raises(AssertionError):
+        sa.spas_sage2_attn_meansim_topk_cuda(q, q, q, tensor_layout="BHND")
+    q = torch.zeros(1, 2, 128, 64, dtype=torch.float16)
+    with pytest.raises(RuntimeError, match="GPU"):          # no silent CPU fallback
+        sa.spas_sage2_attn_meansim_topk_cuda(q, q, q)
+    with pytest.raises(RuntimeError, match="GPU"):
+        sa.block_sparse_sage2_attn_cuda(q, q, q, mask_id=torch.ones(1, 2, 1, 2))
+
+
+def test_block_map_to_mask():
+    m = torch.tensor([[[[1, 0], [0, 1]]]])
+    t = utils.block_map_to_mask(m)
+    assert t.shape == (1, 1, 256, 128)
+    assert t[0, 0, :128, :64].all() and not t[0, 0, :128, 64:].any() and t[0, 0, 128:, 64:].all()
+
+
+def test_workload_generators_shapes_and_determinism():
+    for name, shrink in (("cfg1", None), ("cfg2", dict(B=1, H=2, N=512)), ("cfg3", dict(H=2, grid=(3, 6, 9), text_tokens=30)),
+                         ("cfg4", dict(H=2, N=1024)), ("cfg5", dict(H=1, grid=(2, 8, 11)))):
+        cfg = W.CONFIGS[name]
+        q, k, v = W.make_qkv(cfg, shrink=shrink)
+        q2, _, _ = W.make_qkv(cfg, shrink=shrink)
+        assert torch.equal(q, q2) and q.dtype == cfg.dtype and q.shape == k.shape == v.shape
+        assert q.shape[-1] == cfg.D and torch.isfinite(q.float()).all()
+        assert 0.3 < q.float().std() < 3.0
+    m = W.make_mask_id(W.CONFIGS["cfg2"], 1, 2, 1024)
+    assert m.shape == (1, 2, 8, 16)
+    i = torch.arange(8)
+    assert m[:, :, i, 2 * i].all() and m[:, :, i, 2 * i + 1].all()
+    assert 0.25 < m.float().mean() < 0.5
