@@ -39,11 +39,11 @@ def parse():
 
 
 def cpu_baseline(cfg):
-    """numpy oracle on a bounded sample of the headline workload: one head, N = 4096."""
+    """numpy oracle on a bounded sample of the headline workload: one of its heads at full sequence length."""
     import numpy as np
     from oracle import api as oapi
     from spargeattn_amd import workloads as W
-    n = 4096
+    n = cfg.N if cfg.N <= 32768 else 32768
     q, k, v = W.make_qkv(cfg, device="cpu", shrink=dict(B=1, H=1, N=n))
     qn, kn, vn = (t.float().numpy() for t in (q, k, v))
     tag = "bf16" if cfg.dtype == torch.bfloat16 else "fp16"
