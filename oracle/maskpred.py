@@ -51,8 +51,7 @@ _LN2_HI = F64(0.6931471803691238)      # upper 33 bits of ln 2
 _LN2_LO = F64(1.9082149292705877e-10)  # ln 2 - _LN2_HI
 _EXP_COEF = [F64(1.0) / F64(np.prod(np.arange(1, n + 1, dtype=np.float64))) if n else F64(1.0) for n in range(14)]
 _EXP_MIN = F64(-700.0)
-SUM_LANES = 256  # width of the fixed summation tree (one GPU workgroup)
-WAVE = 64
+WAVE = 64         # width of the fixed summation tree (one GPU wavefront)
 
 
 def cexp(t):
@@ -73,32 +72,33 @@ def cexp(t):
     return np.where(t >= _EXP_MIN, y, 0.0)
 
 
+def _butterfly(acc, width):
+    """xor-butterfly over the last axis (offsets width/2 .. 1); every lane ends with the same value."""
+    idx = np.arange(width)
+    off = width // 2
+    while off >= 1:
+        acc = acc + acc[..., idx ^ off]
+        off //= 2
+    return acc[..., 0]
+
+
 def tree_sum(e):
     """Sum along the last axis with the fixed tree the GPU kernel uses.
 
-    Lane l of 256 adds elements l, l+256, ... in ascending order; each group
-    of 64 lanes is reduced by an xor-butterfly (offsets 32,16,8,4,2,1); the four
-    wave totals are added left to right.
+    Lane l of 64 adds elements l, l+64, ... in ascending order; the 64 partial sums are combined by an
+    xor-butterfly (offsets 32,16,8,4,2,1).
     """
     e = np.asarray(e, dtype=F64)
     n = e.shape[-1]
-    nchunk = (n + SUM_LANES - 1) // SUM_LANES
-    pad = nchunk * SUM_LANES - n
+    nchunk = (n + WAVE - 1) // WAVE
+    pad = nchunk * WAVE - n
     if pad:
         e = np.concatenate([e, np.zeros(e.shape[:-1] + (pad,), dtype=F64)], axis=-1)
-    e = e.reshape(e.shape[:-1] + (nchunk, SUM_LANES))
-    acc = np.zeros(e.shape[:-2] + (SUM_LANES,), dtype=F64)
+    e = e.reshape(e.shape[:-1] + (nchunk, WAVE))
+    acc = np.zeros(e.shape[:-2] + (WAVE,), dtype=F64)
     for c in range(nchunk):
         acc = acc + e[..., c, :]
-    acc = acc.reshape(acc.shape[:-1] + (SUM_LANES // WAVE, WAVE))
-    idx = np.arange(WAVE)
-    for off in (32, 16, 8, 4, 2, 1):
-        acc = acc + acc[..., idx ^ off]
-    w = acc[..., 0]
-    tot = w[..., 0]
-    for i in range(1, SUM_LANES // WAVE):
-        tot = tot + w[..., i]
-    return tot
+    return _butterfly(acc, WAVE)
 
 
 def softmax_T(score, dtype):
@@ -206,14 +206,21 @@ def pool_sim_quant(x, km, bs, simthreshd1, dtype, with_pool=True):
 # --------------------------------------------------------------------------
 
 def pooled_scores(pool_q, pool_k, dtype):
-    """(pooledQ @ pooledK^T) -> T, then * fp32(D**-0.5) -> T (utils.py:388)."""
+    """(pooledQ @ pooledK^T) -> T, then * fp32(D**-0.5) -> T (utils.py:388).
+
+    Fixed order of the dot product: D/8 lanes, lane g adds the products of d = 8g .. 8g+7 in order, the partial
+    sums are combined by an xor-butterfly.  (Products of two T values are exact in binary64.)
+    """
     pq = np.asarray(pool_q, dtype=F64)
     pk = np.asarray(pool_k, dtype=F64)
     d = pq.shape[-1]
-    acc = np.zeros(pq.shape[:-1] + (pk.shape[-2],), dtype=F64)
-    for i in range(d):                                    # fixed order d = 0..D-1
-        acc = acc + pq[..., :, i, None] * pk[..., None, :, i]
-    s1 = round_to(acc, dtype)
+    g = d // 8
+    pq = pq.reshape(pq.shape[:-1] + (g, 8))
+    pk = pk.reshape(pk.shape[:-1] + (g, 8))
+    acc = np.zeros(pq.shape[:-2] + (pk.shape[-3], g), dtype=F64)          # (..., nq, nk, g)
+    for e in range(8):
+        acc = acc + pq[..., :, None, :, e] * pk[..., None, :, :, e]
+    s1 = round_to(_butterfly(acc, g), dtype)
     return round_to(s1.astype(F64) * F64(F32(d ** -0.5)), dtype)
 
 

@@ -40,7 +40,9 @@ def _prologue(q, k, v, tensor_layout):
     qk_dtype = torch.bfloat16 if q.dtype == torch.bfloat16 else torch.float16
     q = q.contiguous().to(qk_dtype)
     k = k.contiguous().to(qk_dtype)
-    v = v.contiguous().to(torch.float16)       # V is always quantised from fp16 (core.py:117)
+    # V is always quantised from fp16 (core.py:117).  A bf16 V is handed over as it is: the quantisation kernel
+    # rounds each element to fp16 in registers, which gives the same values without a pass over HBM.
+    v = v.contiguous() if v.dtype in (torch.float16, torch.bfloat16) else v.contiguous().to(torch.float16)
     return q, k, v
 
 

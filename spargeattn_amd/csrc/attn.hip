@@ -16,8 +16,9 @@
 //    32 scores a lane holds belong to 32 CONSECUTIVE keys (32*half .. 32*half+31): packing them to e4m3 gives the
 //    B operand of the PV MFMA with no shuffle, and the matching A operand is 32 contiguous bytes of a V^T row;
 //  * V lives in HBM as [nk][D][64] e4m3 tiles (one contiguous 64*D-byte read per block), K as (N,D) int8 rows;
-//  * K/V tiles are double-buffered in LDS, the next block's tiles are fetched into VGPRs while the current block
-//    is being computed;
+//  * K/V tiles go through a 3-deep LDS ring: the tiles of block it+2 are in flight from HBM/L2 into VGPRs and the
+//    tiles of block it+1 are written to LDS while block it is being computed, so that ONE workgroup barrier per
+//    block covers both the tile hand-over and the workgroup-wide PV-skip vote;
 //  * workgroup ids are remapped so that one XCD (one L2) works on one head at a time, heaviest rows first.
 #include "common.h"
 #include "launch.h"
@@ -53,8 +54,9 @@ __global__ __launch_bounds__(256, 2) void block_sparse_attn_kernel(const AttnPar
   constexpr int KSTR = D + 16;      // LDS row stride of a K tile (bytes)
   constexpr int VSTR = 64 + 16;     // LDS row stride of a V^T tile (bytes)
   constexpr int CH = D / 64;        // 16-byte chunks per thread per tile (K: 64*D/16/256, V: D*64/16/256)
-  __shared__ __align__(16) int8_t sK[2][64 * KSTR];
-  __shared__ __align__(16) uint8_t sV[2][D * VSTR];
+  constexpr int NBUF = 3;
+  __shared__ __align__(16) int8_t sK[NBUF][64 * KSTR];
+  __shared__ __align__(16) uint8_t sV[NBUF][D * VSTR];
   __shared__ float sRed[2][4];
 
   // ---- workgroup -> (batch*head, q block): one XCD per head at a time, heavy (late) rows first ----------
@@ -87,25 +89,34 @@ __global__ __launch_bounds__(256, 2) void block_sparse_attn_kernel(const AttnPar
   const float c = p.sm_scale_log2;
   const float thr = p.pvthr[head];
 
+  // per-thread 16-byte chunks of a tile: chunk ci = tid + 256*u
   uint4 kr[CH], vr[CH];
-  auto fetch = [&](int blk) {
+  int krow[CH], kcol[CH];
 #pragma unroll
-    for (int u = 0; u < CH; u++) {
-      const int ci = tid + 256 * u;
-      const int row = ci / (D / 16), col = ci % (D / 16);
-      kr[u] = make_uint4(0, 0, 0, 0);
-      if (blk * 64 + row < N) kr[u] = *(const uint4 *)(kbase + ((size_t)blk * 64 + row) * D + col * 16);
-      vr[u] = *(const uint4 *)(vbase + (size_t)blk * (D * 64) + (size_t)ci * 16);
-    }
-  };
-  auto stash = [&](int buf) {
-#pragma unroll
-    for (int u = 0; u < CH; u++) {
-      const int ci = tid + 256 * u;
-      *(uint4 *)(sK[buf] + (ci / (D / 16)) * KSTR + (ci % (D / 16)) * 16) = kr[u];
-      *(uint4 *)(sV[buf] + (ci >> 2) * VSTR + (ci & 3) * 16) = vr[u];
-    }
-  };
+  for (int u = 0; u < CH; u++) {
+    const int ci = tid + 256 * u;
+    krow[u] = ci / (D / 16);
+    kcol[u] = (ci % (D / 16)) * 16;
+  }
+#define SPG_FETCH(BLK)                                                                                    \
+  {                                                                                                       \
+    _Pragma("unroll") for (int u = 0; u < CH; u++) {                                                      \
+      const int grow = (BLK) * 64 + krow[u];                                                              \
+      const int crow = min(grow, N - 1); /* rows beyond N: read a valid row, then zero it */              \
+      uint4 t = *(const uint4 *)(kbase + (size_t)crow * D + kcol[u]);                                     \
+      const uint32_t keep = grow < N ? 0xffffffffu : 0u;                                                  \
+      kr[u] = make_uint4(t.x & keep, t.y & keep, t.z & keep, t.w & keep);                                 \
+      vr[u] = *(const uint4 *)(vbase + (size_t)(BLK) * (D * 64) + (size_t)(tid + 256 * u) * 16);          \
+    }                                                                                                     \
+  }
+#define SPG_STASH(BUF)                                                                                    \
+  {                                                                                                       \
+    _Pragma("unroll") for (int u = 0; u < CH; u++) {                                                      \
+      const int ci = tid + 256 * u;                                                                       \
+      *(uint4 *)(sK[BUF] + krow[u] * KSTR + kcol[u]) = kr[u];                                             \
+      *(uint4 *)(sV[BUF] + (ci >> 2) * VSTR + (ci & 3) * 16) = vr[u];                                     \
+    }                                                                                                     \
+  }
 
   // MFMA row i of key tile kt carries key 32*((i>>2)&1) + 16*kt + 4*(i>>3) + (i&3)
   const int krow0 = 32 * ((r >> 2) & 1) + 4 * (r >> 3) + (r & 3);
@@ -119,14 +130,18 @@ __global__ __launch_bounds__(256, 2) void block_sparse_attn_kernel(const AttnPar
     for (int e = 0; e < 16; e++) O[dt][e] = 0.f;
   int cnt = 0;
 
-  int blk = lut_row[0];
-  fetch(blk);
-  stash(0);
+  int blk = lut_row[0];        // block computed in the current iteration
+  SPG_FETCH(blk);
+  SPG_STASH(0);
+  int blk_next = blk;          // block whose tiles sit in kr/vr
+  if (nv > 1) {
+    blk_next = blk + lut_row[1];
+    SPG_FETCH(blk_next);
+  }
+  __syncthreads();
   int buf = 0;
 
   for (int it = 0; it < nv; it++) {
-    __syncthreads();   // tiles of block `it` are in sK/sV[buf]
-
     // ---- S^T = K . Q^T ---------------------------------------------------------------------------------
     v16i S0, S1;
 #pragma unroll
@@ -139,11 +154,16 @@ __global__ __launch_bounds__(256, 2) void block_sparse_attn_kernel(const AttnPar
       S1 = __builtin_amdgcn_mfma_i32_32x32x32_i8(a1, qreg[ks], S1, 0, 0, 0);
     }
 
+    // ---- ring: tiles of block it+1 (in VGPRs since the previous iteration) -> LDS; fetch block it+2 -------
     const int cur = blk;
-    const bool more = it + 1 < nv;
-    if (more) {
-      blk = cur + lut_row[it + 1];
-      fetch(blk);
+    const int nbuf = buf == NBUF - 1 ? 0 : buf + 1;
+    if (it + 1 < nv) {
+      SPG_STASH(nbuf);
+      blk = blk_next;
+      if (it + 2 < nv) {
+        blk_next = blk + lut_row[it + 2];
+        SPG_FETCH(blk_next);
+      }
     }
 
     const float dq = qs * kscale[cur];
@@ -161,15 +181,16 @@ __global__ __launch_bounds__(256, 2) void block_sparse_attn_kernel(const AttnPar
       a = c * dq;
       fm = (float)imax * a;
     } else {
+      // slot e of this lane is key 64*cur + 32*hh + e; keys beyond `lim` are masked
       const int key0 = cur * 64 + 32 * hh;
-      const bool last = it == nv - 1;
+      int lim = 0x7fffffff;
+      if (p.is_causal) lim = q_row - key0;                       // key > query (attn_utils.cuh:334-361)
+      if (it == nv - 1) lim = min(lim, N - 1 - key0);            // key >= kv_len (attn_utils.cuh:363-389)
       fm = SPG_NEG_BIG;
 #pragma unroll
       for (int e = 0; e < 32; e++) {
         float v = (float)(e < 16 ? S0[e] : S1[e - 16]) * dq;
-        const int key = key0 + e;
-        if (p.is_causal && key > q_row) v = SPG_NEG_BIG;
-        if (last && key >= N) v = SPG_NEG_BIG;
+        v = e > lim ? SPG_NEG_BIG : v;
         x[e] = v;
         fm = fmaxf(fm, v);
       }
@@ -185,7 +206,7 @@ __global__ __launch_bounds__(256, 2) void block_sparse_attn_kernel(const AttnPar
       const float wd = wave_max_f32(diff);
       if (lane == 0) sRed[it & 1][wave] = wd;
     }
-    __syncthreads();   // everyone is done with sK[buf]; sRed is visible
+    __syncthreads();   // block it+1's tiles are in LDS; sRed is visible; ring slot of block it-1 is free
     bool compute = true;
     if (!tail) {
       const float wg = fmaxf(fmaxf(sRed[it & 1][0], sRed[it & 1][1]), fmaxf(sRed[it & 1][2], sRed[it & 1][3]));
@@ -224,9 +245,10 @@ __global__ __launch_bounds__(256, 2) void block_sparse_attn_kernel(const AttnPar
         O[dt] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(av, pb, O[dt], 0, 0, 0, 0, 0, 0);
       }
     }
-    if (more) stash(buf ^ 1);
-    buf ^= 1;
+    buf = nbuf;
   }
+#undef SPG_FETCH
+#undef SPG_STASH
 
   if (p.pv_count != nullptr && tid == 0) p.pv_count[(size_t)bh * p.nq + qb] = cnt;
 

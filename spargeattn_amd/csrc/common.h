@@ -56,10 +56,10 @@ template <> __device__ __forceinline__ uint16_t f32_to_elem<0>(float x) {
   return __builtin_bit_cast(uint16_t, h);
 }
 template <> __device__ __forceinline__ uint16_t f32_to_elem<1>(float x) {
-  uint32_t u = __builtin_bit_cast(uint32_t, x);
-  if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x40);
-  u += 0x7fffu + ((u >> 16) & 1u);
-  return (uint16_t)(u >> 16);
+  const uint32_t u = __builtin_bit_cast(uint32_t, x);
+  const uint32_t rounded = (u + 0x7fffu + ((u >> 16) & 1u)) >> 16;
+  const uint32_t quiet = (u >> 16) | 0x40u;
+  return (uint16_t)(((u & 0x7fffffffu) > 0x7f800000u) ? quiet : rounded);   // select, no branch
 }
 
 // ---------------------------------------------------------------------------------------------

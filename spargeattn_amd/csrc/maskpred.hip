@@ -58,6 +58,7 @@ template <int DT>
 __global__ void km_final_kernel(const double *__restrict__ part, uint16_t *__restrict__ km, int nchunk, int D, int N) {
   const int bh = blockIdx.x, d = threadIdx.x;
   double s = 0.0;
+#pragma unroll 16
   for (int i = 0; i < nchunk; i++) s += part[((size_t)bh * nchunk + i) * D + d];
   km[(size_t)bh * D + d] = f64_to_elem<DT>(s / (double)N);
 }
@@ -216,18 +217,20 @@ __device__ __forceinline__ double cexp(double t) {
 }
 
 // exclusive prefix of per-thread counts over the 256 threads of the workgroup; returns (offset, total)
-__device__ __forceinline__ int2 block_exclusive_scan_i32(int v, int *s_tmp /* >= 256 ints */) {
-  const int tid = threadIdx.x;
-  s_tmp[tid] = v;
-  __syncthreads();
-  int off = 0, tot = 0;
-  for (int u = 0; u < 256; u++) {
-    const int w = s_tmp[u];
-    off += (u < tid) ? w : 0;
-    tot += w;
+__device__ __forceinline__ int2 block_exclusive_scan_i32(int v, int *s_tmp /* >= 4 ints */) {
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  int inc = v;
+#pragma unroll
+  for (int o = 1; o < 64; o <<= 1) {
+    const int t = __shfl_up(inc, o, SPG_WAVE);
+    if (lane >= o) inc += t;
   }
+  __syncthreads();                       // s_tmp may still be read from a previous call
+  if (lane == 63) s_tmp[wave] = inc;
   __syncthreads();
-  return make_int2(off, tot);
+  const int w0 = s_tmp[0], w1 = s_tmp[1], w2 = s_tmp[2], w3 = s_tmp[3];
+  const int base = (wave > 0 ? w0 : 0) + (wave > 1 ? w1 : 0) + (wave > 2 ? w2 : 0);
+  return make_int2(base + inc - v, w0 + w1 + w2 + w3);
 }
 
 // flags (per column, via functor) -> ascending compact index list -> delta LUT, zero tail, valid count.
@@ -257,7 +260,7 @@ __device__ __forceinline__ void emit_lut(FlagFn flag, int nk, int nkp, int32_t *
 // dynamic LDS: 12 * nkp bytes (nkp = power of two >= max(nk, 256)).
 // =============================================================================================
 template <int D, int DT>
-__global__ __launch_bounds__(256) void block_select_kernel(
+__global__ __launch_bounds__(256, 4) void block_select_kernel(
     const uint16_t *__restrict__ pool_q, const uint8_t *__restrict__ sim_q, const uint16_t *__restrict__ pool_k,
     const uint8_t *__restrict__ sim_k, const float *__restrict__ topk, const float *__restrict__ cdfthr, int is_causal,
     int sink, int32_t *__restrict__ lut, int32_t *__restrict__ valid, uint8_t *__restrict__ bmap, int H, int nq, int nk,
@@ -284,45 +287,58 @@ __global__ __launch_bounds__(256) void block_select_kernel(
   const uint8_t *simk = sim_k + (size_t)bh * nk;
   float *s_score = (float *)okey;
 
-  // ---- scores (fixed order d = 0..D-1), two roundings to the input dtype, masks --------------------
-  float lmax = -INFINITY;
-  for (int j = tid; j < nk; j += 256) {
-    const uint4 *row = (const uint4 *)(pk_base + (size_t)j * D);
-    double acc = 0.0;
+  // ---- scores: G = D/8 lanes share one column (one coalesced 16-byte load each); a lane adds its 8 products
+  //      in order, the G partial sums are combined by an xor butterfly (offsets G/2 .. 1).  Two roundings to the
+  //      input dtype, then the masks.
+  constexpr int G = D / 8;
+  const int g = tid % G, cg = tid / G;
+  float pqv[8];
 #pragma unroll
-    for (int cch = 0; cch < D / 8; cch++) {
-      const uint4 v = row[cch];
+  for (int e = 0; e < 8; e++) pqv[e] = s_pq[g * 8 + e];
+  float lmax = -INFINITY;
+  for (int j0 = 0; j0 < nk; j0 += 256 / G) {
+    const int j = j0 + cg;
+    double acc = 0.0;
+    if (j < nk) {
+      const uint4 v = *(const uint4 *)(pk_base + (size_t)j * D + g * 8);
       const uint32_t w[4] = {v.x, v.y, v.z, v.w};
 #pragma unroll
       for (int e = 0; e < 8; e++) {
         const float kf = elem_to_f32<DT>((uint16_t)((e & 1) ? (w[e >> 1] >> 16) : (w[e >> 1] & 0xffffu)));
-        acc = acc + (double)s_pq[cch * 8 + e] * (double)kf;   // product exact in binary64
+        acc = acc + (double)pqv[e] * (double)kf;   // product exact in binary64
       }
     }
-    const float s1 = elem_to_f32<DT>(f64_to_elem<DT>(acc));
-    float s2 = elem_to_f32<DT>(f64_to_elem<DT>((double)s1 * (double)sm_scale));
-    if (!simk[j] || j >= causal_lim) s2 = -INFINITY;
-    s_score[j] = s2;
-    lmax = fmaxf(lmax, s2);
+#pragma unroll
+    for (int o = G / 2; o >= 1; o >>= 1) acc = acc + shfl_xor_f64(acc, o);
+    if (g == 0 && j < nk) {
+      const float s1 = elem_to_f32<DT>(f64_to_elem<DT>(acc));
+      float s2 = elem_to_f32<DT>(f64_to_elem<DT>((double)s1 * (double)sm_scale));
+      if (!simk[j] || j >= causal_lim) s2 = -INFINITY;
+      s_score[j] = s2;
+      lmax = fmaxf(lmax, s2);
+    }
   }
   lmax = wave_max_f32(lmax);
   if ((tid & 63) == 0) s_wmax[tid >> 6] = lmax;
   __syncthreads();
   const float mx = fmaxf(fmaxf(s_wmax[0], s_wmax[1]), fmaxf(s_wmax[2], s_wmax[3]));
 
-  // ---- exp and the fixed summation tree -------------------------------------------------------------
-  double part = 0.0;
+  // ---- exp, then the fixed summation tree: lane l of ONE wavefront adds e[l], e[l+64], ... in order, followed
+  //      by an xor butterfly (32 .. 1) ------------------------------------------------------------------------
   for (int j = tid; j < nk; j += 256) {
     const float s2 = s_score[j];
-    const double e = (s2 == -INFINITY) ? 0.0 : cexp((double)s2 - (double)mx);
-    e_buf[j] = e;
-    part = part + e;
+    e_buf[j] = (s2 == -INFINITY) ? 0.0 : cexp((double)s2 - (double)mx);
   }
-#pragma unroll
-  for (int o = 32; o >= 1; o >>= 1) part = part + shfl_xor_f64(part, o);
-  if ((tid & 63) == 0) s_wsum[tid >> 6] = part;
   __syncthreads();
-  const double total = ((s_wsum[0] + s_wsum[1]) + s_wsum[2]) + s_wsum[3];
+  if (tid < 64) {
+    double part = 0.0;
+    for (int j = tid; j < nk; j += 64) part = part + e_buf[j];
+#pragma unroll
+    for (int o = 32; o >= 1; o >>= 1) part = part + shfl_xor_f64(part, o);
+    if (tid == 0) s_wsum[0] = part;
+  }
+  __syncthreads();
+  const double total = s_wsum[0];
 
   // ---- probabilities -> sortable keys (value bits, then lower index first) --------------------------
   for (int j = tid; j < nk; j += 256) {
