@@ -78,8 +78,9 @@ int spg_map_to_lut(const void *mask, int mask_kind, int32_t *lut, int32_t *valid
  * (csrc/fused/fused.cu:193-267, 269-344; called at core.py:147,151).
  * v (B,H,N,D) dtype (bf16 input is first rounded to fp16, core.py:117).
  * out: v8 e4m3fn codes in TILE layout [B][H][nk][D][64] (key index fastest inside a 64-key tile, rows
- *      beyond N are zero) - the layout the attention kernel's V^T operand reads; v_scale (B,H,D) float32
- *      = amax/2.25.  v_scale doubles as the amax scratch between the passes. */
+ *      beyond N are zero; inside a 64-byte row the four 16-key chunks are XOR-swizzled: key chunk kc is
+ *      stored at slot kc ^ ((d >> 1) & 3)) - the layout the attention kernel copies to LDS verbatim;
+ *      v_scale (B,H,D) float32 = amax/2.25.  v_scale doubles as the amax scratch between the passes. */
 int spg_v_quant_fp8(const void *v, uint8_t *v8, float *v_scale, int B, int H, int N, int D, int dtype,
                     void *stream);
 

@@ -163,6 +163,31 @@ def v_quant_fp8(v):
     return v8, v_scale
 
 
+def _v_swizzle_index(D, device):
+    """slot index (D,4) such that tile[d, slot] holds key chunk slot ^ ((d >> 1) & 3)."""
+    d = torch.arange(D, device=device)
+    return torch.arange(4, device=device)[None, :] ^ ((d >> 1) & 3)[:, None]
+
+
+def v8_tiles_to_natural(v8):
+    """(B,H,nk,D,64) swizzled tile layout -> (B,H,nk*64,D) codes in natural key order."""
+    B, H, nk, D, _ = v8.shape
+    idx = _v_swizzle_index(D, v8.device)                       # natural chunk kc sits at slot kc ^ swz = idx[d, kc]
+    t = v8.view(B, H, nk, D, 4, 16)
+    nat = torch.gather(t, 4, idx.view(1, 1, 1, D, 4, 1).expand(B, H, nk, D, 4, 16))
+    return nat.reshape(B, H, nk, D, 64).permute(0, 1, 2, 4, 3).reshape(B, H, nk * 64, D)
+
+
+def v8_natural_to_tiles(v8_nat):
+    """(B,H,nk*64,D) codes in natural key order -> the (B,H,nk,D,64) swizzled tile layout the attention kernel reads."""
+    B, H, n64, D = v8_nat.shape
+    nk = n64 // 64
+    t = v8_nat.view(B, H, nk, 64, D).permute(0, 1, 2, 4, 3).contiguous().view(B, H, nk, D, 4, 16)
+    idx = _v_swizzle_index(D, v8_nat.device)                   # slot s holds chunk s ^ swz = idx[d, s]
+    sw = torch.gather(t, 4, idx.view(1, 1, 1, D, 4, 1).expand(B, H, nk, D, 4, 16))
+    return sw.reshape(B, H, nk, D, 64).contiguous()
+
+
 def block_sparse_attn(q8, k8, v8, out, lut, valid, pvthreshd, q_scale, k_scale, v_scale, sm_scale,
                       is_causal=False, return_pv_count=False):
     _dev(q8, k8, v8, out, lut, valid, pvthreshd, q_scale, k_scale, v_scale)

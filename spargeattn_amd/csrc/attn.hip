@@ -16,9 +16,11 @@
 //    32 scores a lane holds belong to 32 CONSECUTIVE keys (32*half .. 32*half+31): packing them to e4m3 gives the
 //    B operand of the PV MFMA with no shuffle, and the matching A operand is 32 contiguous bytes of a V^T row;
 //  * V lives in HBM as [nk][D][64] e4m3 tiles (one contiguous 64*D-byte read per block), K as (N,D) int8 rows;
-//  * K/V tiles go through a 3-deep LDS ring: the tiles of block it+2 are in flight from HBM/L2 into VGPRs and the
-//    tiles of block it+1 are written to LDS while block it is being computed, so that ONE workgroup barrier per
-//    block covers both the tile hand-over and the workgroup-wide PV-skip vote;
+//  * K/V tiles go HBM/L2 -> LDS directly (global_load_lds_dwordx4, no VGPR staging) through a 3-deep LDS ring:
+//    the tiles of block it+2 are in flight while block it is computed, and ONE workgroup barrier per block covers
+//    both the tile hand-over and the workgroup-wide PV-skip vote;
+//  * LDS tiles are unpadded; bank conflicts are avoided by an XOR swizzle of the 16-byte chunks inside a row
+//    (applied to the per-lane global address for K, baked into the HBM tile layout for V);
 //  * workgroup ids are remapped so that one XCD (one L2) works on one head at a time, heaviest rows first.
 #include "common.h"
 #include "launch.h"
@@ -27,6 +29,7 @@ namespace spg {
 
 typedef int v4i __attribute__((ext_vector_type(4)));
 typedef int v8i __attribute__((ext_vector_type(8)));
+typedef int v8i_a16 __attribute__((ext_vector_type(8), aligned(16)));
 typedef int v16i __attribute__((ext_vector_type(16)));
 typedef float v16f __attribute__((ext_vector_type(16)));
 
@@ -47,17 +50,26 @@ struct AttnParams {
   int total_wg, wg_per_xcd;
 };
 
+// 16-byte-chunk swizzles.  K tile row = key (D bytes, D/16 chunks); V^T tile row = channel (64 bytes, 4 chunks).
+// The functions are chosen such that any 8 consecutive lanes of a ds_read_b128 hit 8 different 16-byte bank groups.
+template <int D>
+__device__ __forceinline__ int k_swz(int row) {
+  if constexpr (D == 128) return (row & 3) | (((row >> 5) & 1) << 2);
+  else return ((row >> 1) & 1) | (((row >> 5) & 1) << 1);
+}
+__device__ __forceinline__ int v_swz(int row) { return (row >> 1) & 3; }
+
 template <int D, int ODT>
-__global__ __launch_bounds__(256, 2) void block_sparse_attn_kernel(const AttnParams p) {
+__global__ __launch_bounds__(256, 3) void block_sparse_attn_kernel(const AttnParams p) {
   constexpr int KS = D / 32;        // k-steps of the int8 MFMA
   constexpr int NDT = D / 32;       // 32-channel output tiles
-  constexpr int KSTR = D + 16;      // LDS row stride of a K tile (bytes)
-  constexpr int VSTR = 64 + 16;     // LDS row stride of a V^T tile (bytes)
-  constexpr int CH = D / 64;        // 16-byte chunks per thread per tile (K: 64*D/16/256, V: D*64/16/256)
+  constexpr int TILE = 64 * D;      // bytes of one K tile = bytes of one V^T tile
+  constexpr int CPR = D / 16;       // 16-byte chunks per K row
+  constexpr int WL = D / 64;        // global_load_lds instructions per wave per tile (TILE / 1024 / 4)
   constexpr int NBUF = 3;
-  __shared__ __align__(16) int8_t sK[NBUF][64 * KSTR];
-  __shared__ __align__(16) uint8_t sV[NBUF][D * VSTR];
-  __shared__ float sRed[2][4];
+  __shared__ __align__(1024) unsigned char sK[NBUF][TILE];
+  __shared__ __align__(1024) unsigned char sV[NBUF][TILE];
+  __shared__ int sVote[2][4];
 
   // ---- workgroup -> (batch*head, q block): one XCD per head at a time, heavy (late) rows first ----------
   const int w = blockIdx.x;
@@ -83,43 +95,40 @@ __global__ __launch_bounds__(256, 2) void block_sparse_attn_kernel(const AttnPar
   }
 
   const int8_t *kbase = p.k8 + (size_t)bh * N * D;
-  const uint8_t *vbase = p.v8 + (size_t)bh * p.nk * (size_t)(D * 64);
+  const uint8_t *vbase = p.v8 + (size_t)bh * p.nk * (size_t)TILE;
   const float *kscale = p.k_scale + (size_t)bh * p.nk;
   const float qs = p.q_scale[(size_t)bh * p.nq + qb];
   const float c = p.sm_scale_log2;
   const float thr = p.pvthr[head];
 
-  // per-thread 16-byte chunks of a tile: chunk ci = tid + 256*u
-  uint4 kr[CH], vr[CH];
-  int krow[CH], kcol[CH];
+  // ---- tile loader: wave w copies LDS bytes [1024*(WL*w+u), +1024) of each tile, lane l the 16-byte chunk l ----
+  // K: LDS chunk position pos <-> (row = pos / CPR, slot = pos % CPR) holds global chunk slot ^ k_swz(row).
+  int k_row[WL], k_off[WL];
 #pragma unroll
-  for (int u = 0; u < CH; u++) {
-    const int ci = tid + 256 * u;
-    krow[u] = ci / (D / 16);
-    kcol[u] = (ci % (D / 16)) * 16;
+  for (int u = 0; u < WL; u++) {
+    const int pos = (WL * wave + u) * 64 + lane;
+    k_row[u] = pos / CPR;
+    k_off[u] = ((pos % CPR) ^ k_swz<D>(pos / CPR)) * 16;
   }
-#define SPG_FETCH(BLK)                                                                                    \
-  {                                                                                                       \
-    _Pragma("unroll") for (int u = 0; u < CH; u++) {                                                      \
-      const int grow = (BLK) * 64 + krow[u];                                                              \
-      const int crow = min(grow, N - 1); /* rows beyond N: read a valid row, then zero it */              \
-      uint4 t = *(const uint4 *)(kbase + (size_t)crow * D + kcol[u]);                                     \
-      const uint32_t keep = grow < N ? 0xffffffffu : 0u;                                                  \
-      kr[u] = make_uint4(t.x & keep, t.y & keep, t.z & keep, t.w & keep);                                 \
-      vr[u] = *(const uint4 *)(vbase + (size_t)(BLK) * (D * 64) + (size_t)(tid + 256 * u) * 16);          \
-    }                                                                                                     \
-  }
-#define SPG_STASH(BUF)                                                                                    \
-  {                                                                                                       \
-    _Pragma("unroll") for (int u = 0; u < CH; u++) {                                                      \
-      const int ci = tid + 256 * u;                                                                       \
-      *(uint4 *)(sK[BUF] + krow[u] * KSTR + kcol[u]) = kr[u];                                             \
-      *(uint4 *)(sV[BUF] + (ci >> 2) * VSTR + (ci & 3) * 16) = vr[u];                                     \
-    }                                                                                                     \
+  typedef __attribute__((address_space(3))) void *lds_ptr_t;
+  typedef const __attribute__((address_space(1))) void *glb_ptr_t;
+#define SPG_LOAD_TILES(BLK, BUF)                                                                              \
+  {                                                                                                           \
+    _Pragma("unroll") for (int u = 0; u < WL; u++) {                                                          \
+      /* rows beyond N (last block only) are clamped: their scores are masked, their V rows are zero */       \
+      const int grow = min((BLK) * 64 + k_row[u], N - 1);                                                     \
+      __builtin_amdgcn_global_load_lds((glb_ptr_t)(kbase + (size_t)grow * D + k_off[u]),                      \
+                                       (lds_ptr_t)(sK[BUF] + (WL * wave + u) * 1024), 16, 0, 0);              \
+      __builtin_amdgcn_global_load_lds(                                                                       \
+          (glb_ptr_t)(vbase + (size_t)(BLK) * TILE + (size_t)((WL * wave + u) * 64 + lane) * 16),             \
+          (lds_ptr_t)(sV[BUF] + (WL * wave + u) * 1024), 16, 0, 0);                                           \
+    }                                                                                                         \
   }
 
   // MFMA row i of key tile kt carries key 32*((i>>2)&1) + 16*kt + 4*(i>>3) + (i&3)
   const int krow0 = 32 * ((r >> 2) & 1) + 4 * (r >> 3) + (r & 3);
+  const int ksw0 = k_swz<D>(krow0), ksw1 = k_swz<D>(krow0 + 16);
+  const int vsw = v_swz(r);     // v_swz(32*dt + r) does not depend on dt
 
   float m = SPG_NEG_BIG;
   float dsum = hh == 0 ? 1.0f : 0.0f;     // the two half-lanes of a query share d = 1.0 (sm89.cuh:172)
@@ -131,41 +140,34 @@ __global__ __launch_bounds__(256, 2) void block_sparse_attn_kernel(const AttnPar
   int cnt = 0;
 
   int blk = lut_row[0];        // block computed in the current iteration
-  SPG_FETCH(blk);
-  SPG_STASH(0);
-  int blk_next = blk;          // block whose tiles sit in kr/vr
+  int blk_ld = blk;            // last block whose loads were issued
+  SPG_LOAD_TILES(blk, 0);
   if (nv > 1) {
-    blk_next = blk + lut_row[1];
-    SPG_FETCH(blk_next);
+    blk_ld = blk + lut_row[1];
+    SPG_LOAD_TILES(blk_ld, 1);
   }
-  __syncthreads();
+  int blk_n1 = blk_ld;         // block of iteration it+1
   int buf = 0;
 
   for (int it = 0; it < nv; it++) {
+    if (it == 0) {
+      __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0)
+      __syncthreads();
+    }
     // ---- S^T = K . Q^T ---------------------------------------------------------------------------------
     v16i S0, S1;
 #pragma unroll
     for (int e = 0; e < 16; e++) { S0[e] = 0; S1[e] = 0; }
 #pragma unroll
     for (int ks = 0; ks < KS; ks++) {
-      const v4i a0 = *(const v4i *)(sK[buf] + krow0 * KSTR + 32 * ks + 16 * hh);
-      const v4i a1 = *(const v4i *)(sK[buf] + (krow0 + 16) * KSTR + 32 * ks + 16 * hh);
+      const int ch = 2 * ks + hh;
+      const v4i a0 = *(const v4i *)(sK[buf] + krow0 * D + ((ch ^ ksw0) * 16));
+      const v4i a1 = *(const v4i *)(sK[buf] + (krow0 + 16) * D + ((ch ^ ksw1) * 16));
       S0 = __builtin_amdgcn_mfma_i32_32x32x32_i8(a0, qreg[ks], S0, 0, 0, 0);
       S1 = __builtin_amdgcn_mfma_i32_32x32x32_i8(a1, qreg[ks], S1, 0, 0, 0);
     }
 
-    // ---- ring: tiles of block it+1 (in VGPRs since the previous iteration) -> LDS; fetch block it+2 -------
     const int cur = blk;
-    const int nbuf = buf == NBUF - 1 ? 0 : buf + 1;
-    if (it + 1 < nv) {
-      SPG_STASH(nbuf);
-      blk = blk_next;
-      if (it + 2 < nv) {
-        blk_next = blk + lut_row[it + 2];
-        SPG_FETCH(blk_next);
-      }
-    }
-
     const float dq = qs * kscale[cur];
     const bool tail = it >= nv - 2;   // last two blocks: masks, no PV skip (sm89.cuh:467-648)
     float x[32];
@@ -197,21 +199,26 @@ __global__ __launch_bounds__(256, 2) void block_sparse_attn_kernel(const AttnPar
       a = c;
       fm = fm * c;
     }
-    fm = fmaxf(fm, __shfl_xor(fm, 32, SPG_WAVE));
+    fm = half_swap_max_f32(fm);
     const float diff = fm - m;
     const float m_new = fmaxf(m, fm);
     const float osc = __builtin_amdgcn_exp2f(m - m_new);
     m = m_new;
     if (!tail) {
-      const float wd = wave_max_f32(diff);
-      if (lane == 0) sRed[it & 1][wave] = wd;
+      // max over rows of (diff) + thr > 0  <=>  some row has diff + thr > 0 (fp32 addition is monotonic)
+      const int vote = __any(diff + thr > 0.f);
+      if (lane == 0) sVote[it & 1][wave] = vote;
     }
-    __syncthreads();   // block it+1's tiles are in LDS; sRed is visible; ring slot of block it-1 is free
+    __builtin_amdgcn_s_waitcnt(0x0F70);   // this wave's share of block it+1's tiles has landed in LDS
+    __syncthreads();   // block it+1's tiles are complete; the votes are visible; ring slot of block it-1 is free
+    if (it + 2 < nv) {
+      blk_ld += lut_row[it + 2];
+      const int b2 = buf == 0 ? 2 : buf - 1;   // (it+2) % 3
+      SPG_LOAD_TILES(blk_ld, b2);
+    }
     bool compute = true;
-    if (!tail) {
-      const float wg = fmaxf(fmaxf(sRed[it & 1][0], sRed[it & 1][1]), fmaxf(sRed[it & 1][2], sRed[it & 1][3]));
-      compute = (wg + thr > 0.f);     // workgroup-uniform (PVThresholdMode::kPerBlock, sm89.cuh:318-353)
-    }
+    if (!tail)         // workgroup-uniform (PVThresholdMode::kPerBlock, sm89.cuh:318-353)
+      compute = (sVote[it & 1][0] | sVote[it & 1][1] | sVote[it & 1][2] | sVote[it & 1][3]) != 0;
     dsum *= osc;
     if (__any(osc != 1.0f)) {
 #pragma unroll
@@ -238,22 +245,24 @@ __global__ __launch_bounds__(256, 2) void block_sparse_attn_kernel(const AttnPar
       }
 #pragma unroll
       for (int dt = 0; dt < NDT; dt++) {
-        const uint8_t *vrow = sV[buf] + (32 * dt + r) * VSTR + 32 * hh;
-        const v4i lo = *(const v4i *)(vrow);
-        const v4i hi = *(const v4i *)(vrow + 16);
+        const unsigned char *vrow = sV[buf] + (32 * dt + r) * 64;
+        const v4i lo = *(const v4i *)(vrow + (((2 * hh) ^ vsw) * 16));
+        const v4i hi = *(const v4i *)(vrow + (((2 * hh + 1) ^ vsw) * 16));
         const v8i av = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
         O[dt] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(av, pb, O[dt], 0, 0, 0, 0, 0, 0);
       }
     }
-    buf = nbuf;
+    // advance: block of iteration it+1, then the one after
+    blk = blk_n1;
+    blk_n1 = blk_ld;
+    buf = buf == NBUF - 1 ? 0 : buf + 1;
   }
-#undef SPG_FETCH
-#undef SPG_STASH
+#undef SPG_LOAD_TILES
 
   if (p.pv_count != nullptr && tid == 0) p.pv_count[(size_t)bh * p.nq + qb] = cnt;
 
   // ---- epilogue: O / d * v_scale -> out dtype -----------------------------------------------------------
-  const float dtot = dsum + __shfl_xor(dsum, 32, SPG_WAVE);
+  const float dtot = half_swap_sum_f32(dsum);
   const float inv = __builtin_amdgcn_rcpf(dtot);
   if (q_row < N) {
     uint16_t *orow = (uint16_t *)p.out + ((size_t)bh * N + q_row) * D;

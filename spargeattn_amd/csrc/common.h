@@ -80,6 +80,26 @@ __device__ __forceinline__ long long shfl_xor_i64(long long v, int mask) {
   return (long long)(((uint64_t)hi << 32) | lo);
 }
 
+// Combine the value of lane l with that of lane l^32 (the two 32-lane halves) with one v_permlane32_swap:
+// the instruction exchanges lanes 32..63 of its first register with lanes 0..31 of its second, so that afterwards
+// the first register holds the lower half's values in both halves and the second the upper half's.
+// (Inline asm with two distinct registers: the builtin mis-compiles when both operands are the same value.)
+__device__ __forceinline__ void half_swap(float v, float &lo, float &hi) {
+  lo = v;
+  hi = v;
+  asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1" : "+v"(lo), "+v"(hi));
+}
+__device__ __forceinline__ float half_swap_max_f32(float v) {
+  float lo, hi;
+  half_swap(v, lo, hi);
+  return fmaxf(lo, hi);
+}
+__device__ __forceinline__ float half_swap_sum_f32(float v) {
+  float lo, hi;
+  half_swap(v, lo, hi);
+  return lo + hi;
+}
+
 __device__ __forceinline__ float wave_max_f32(float v) {
 #pragma unroll
   for (int o = 32; o >= 1; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, SPG_WAVE));

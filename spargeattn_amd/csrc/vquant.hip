@@ -1,5 +1,7 @@
 // V path for gfx950: fp16 cast, per-(b,h,channel) absmax, FP8 e4m3 quantisation written straight into the
-// [B][H][nk][D][64] tile layout the attention kernel's V^T operand reads.
+// [B][H][nk][D][64] tile layout the attention kernel's V^T operand reads.  Inside a 64-byte tile row (one channel,
+// 64 keys) the four 16-key chunks are stored XOR-swizzled: key chunk kc sits at slot kc ^ ((d >> 1) & 3), which is
+// the LDS bank-conflict swizzle of the attention kernel baked into the HBM layout (a tile is copied to LDS verbatim).
 // Replaces TransposePadPermuteKernel + MeanScaleKernel (csrc/fused/fused.cu:26-77, 80-191) called with
 // scale_max = 2.25 (spas_sage_attn/core.py:147-151).  HBM-bound: V is read twice (absmax, quantise), written once
 // at 1 B/element.  Compile with -ffp-contract=off.
@@ -89,10 +91,11 @@ __global__ __launch_bounds__(256) void v_quant_kernel(const uint16_t *__restrict
   }
   __syncthreads();
   uint8_t *out = v8 + ((size_t)bh * nk + blk) * (size_t)(D * 64);
-  for (int i = tid; i < D * 4; i += 256) {   // 16-byte pieces: D rows x 4
-    const int d = i >> 2, part = i & 3;
-    const uint32_t *src = (const uint32_t *)(tile + d * LDW + part * 16);
-    *(uint4 *)(out + d * 64 + part * 16) = make_uint4(src[0], src[1], src[2], src[3]);
+  for (int i = tid; i < D * 4; i += 256) {   // 16-byte pieces: D rows x 4 slots
+    const int d = i >> 2, slot = i & 3;
+    const int kc = slot ^ ((d >> 1) & 3);      // key chunk stored in this slot
+    const uint32_t *src = (const uint32_t *)(tile + d * LDW + kc * 16);
+    *(uint4 *)(out + d * 64 + slot * 16) = make_uint4(src[0], src[1], src[2], src[3]);
   }
 }
 

@@ -23,8 +23,8 @@ def bits_equal_T(t_gpu, ref_np, dtype):
 
 def v8_natural(v8_tiles, n_rows=None):
     """(B,H,nk,D,64) tile layout -> (B,H,nk*64,D) natural order (numpy uint8)."""
-    B, H, nk, D, _ = v8_tiles.shape
-    nat = v8_tiles.permute(0, 1, 2, 4, 3).reshape(B, H, nk * 64, D).cpu().numpy()
+    from spargeattn_amd import _lib
+    nat = _lib.v8_tiles_to_natural(v8_tiles).cpu().numpy()
     return nat if n_rows is None else nat[:, :, :n_rows]
 
 

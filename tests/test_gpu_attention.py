@@ -45,7 +45,7 @@ def _run_kernel_on_oracle_tensors(res, out_dtype, H, N, D, pvthreshd, is_causal=
     B = q8.shape[0]
     nk = (N + 63) // 64
     v8_nat = torch.from_numpy(res["v8"][:, :, :nk * 64]).to(dev)            # (B,H,nk*64,D)
-    v8 = v8_nat.view(B, H, nk, 64, D).permute(0, 1, 2, 4, 3).contiguous()  # tile layout
+    v8 = _lib.v8_natural_to_tiles(v8_nat)                                   # tile layout
     out = torch.zeros((B, H, N, D), dtype=out_dtype, device=dev)
     pvt = torch.full((H,), float(pvthreshd), dtype=torch.float32, device=dev)
     pvc = _lib.block_sparse_attn(q8, k8, v8, out, torch.from_numpy(res["lut"]).to(dev),
