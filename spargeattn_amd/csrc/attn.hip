@@ -103,25 +103,34 @@ __global__ __launch_bounds__(256, 3) void block_sparse_attn_kernel(const AttnPar
 
   // ---- tile loader: wave w copies LDS bytes [1024*(WL*w+u), +1024) of each tile, lane l the 16-byte chunk l ----
   // K: LDS chunk position pos <-> (row = pos / CPR, slot = pos % CPR) holds global chunk slot ^ k_swz(row).
-  int k_row[WL], k_off[WL];
+  // A tile's global address is (uniform base of the block) + (per-lane 32-bit offset): no per-load VALU work.
+  uint32_t k_lane[WL], v_lane[WL];
 #pragma unroll
   for (int u = 0; u < WL; u++) {
     const int pos = (WL * wave + u) * 64 + lane;
-    k_row[u] = pos / CPR;
-    k_off[u] = ((pos % CPR) ^ k_swz<D>(pos / CPR)) * 16;
+    k_lane[u] = (uint32_t)((pos / CPR) * D + ((pos % CPR) ^ k_swz<D>(pos / CPR)) * 16);
+    v_lane[u] = (uint32_t)pos * 16u;
   }
+  const int last_partial_blk = (N % 64) ? p.nk - 1 : -1;   // the only block with rows beyond N
   typedef __attribute__((address_space(3))) void *lds_ptr_t;
   typedef const __attribute__((address_space(1))) void *glb_ptr_t;
 #define SPG_LOAD_TILES(BLK, BUF)                                                                              \
   {                                                                                                           \
+    const int8_t *kb_ = kbase + (size_t)(BLK) * TILE;                                                         \
+    const uint8_t *vb_ = vbase + (size_t)(BLK) * TILE;                                                        \
+    const int rows_ok_ = N - (BLK) * 64; /* >= 64 except in the partial last block */                         \
     _Pragma("unroll") for (int u = 0; u < WL; u++) {                                                          \
-      /* rows beyond N (last block only) are clamped: their scores are masked, their V rows are zero */       \
-      const int grow = min((BLK) * 64 + k_row[u], N - 1);                                                     \
-      __builtin_amdgcn_global_load_lds((glb_ptr_t)(kbase + (size_t)grow * D + k_off[u]),                      \
-                                       (lds_ptr_t)(sK[BUF] + (WL * wave + u) * 1024), 16, 0, 0);              \
-      __builtin_amdgcn_global_load_lds(                                                                       \
-          (glb_ptr_t)(vbase + (size_t)(BLK) * TILE + (size_t)((WL * wave + u) * 64 + lane) * 16),             \
-          (lds_ptr_t)(sV[BUF] + (WL * wave + u) * 1024), 16, 0, 0);                                           \
+      uint32_t ko_ = k_lane[u];                                                                               \
+      if ((BLK) == last_partial_blk) {                                                                        \
+        /* rows beyond N are clamped to row N-1: their scores are masked, their V rows are zero */            \
+        const int pos = (WL * wave + u) * 64 + lane;                                                          \
+        const int row_ = min(pos / CPR, rows_ok_ - 1);                                                        \
+        ko_ = (uint32_t)(row_ * D + ((pos % CPR) ^ k_swz<D>(pos / CPR)) * 16);                                \
+      }                                                                                                       \
+      __builtin_amdgcn_global_load_lds((glb_ptr_t)(kb_ + ko_), (lds_ptr_t)(sK[BUF] + (WL * wave + u) * 1024), \
+                                       16, 0, 0);                                                             \
+      __builtin_amdgcn_global_load_lds((glb_ptr_t)(vb_ + v_lane[u]),                                          \
+                                       (lds_ptr_t)(sV[BUF] + (WL * wave + u) * 1024), 16, 0, 0);              \
     }                                                                                                         \
   }
 
@@ -139,16 +148,17 @@ __global__ __launch_bounds__(256, 3) void block_sparse_attn_kernel(const AttnPar
     for (int e = 0; e < 16; e++) O[dt][e] = 0.f;
   int cnt = 0;
 
-  int blk = lut_row[0];        // block computed in the current iteration
-  int blk_ld = blk;            // last block whose loads were issued
+  int blk = __builtin_amdgcn_readfirstlane(lut_row[0]);   // block computed in the current iteration
+  int blk_ld = blk;                                         // last block whose loads were issued
   SPG_LOAD_TILES(blk, 0);
   if (nv > 1) {
-    blk_ld = blk + lut_row[1];
+    blk_ld = __builtin_amdgcn_readfirstlane(blk + lut_row[1]);
     SPG_LOAD_TILES(blk_ld, 1);
   }
   int blk_n1 = blk_ld;         // block of iteration it+1
   int buf = 0;
 
+#pragma unroll 1
   for (int it = 0; it < nv; it++) {
     if (it == 0) {
       __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0)
@@ -212,7 +222,7 @@ __global__ __launch_bounds__(256, 3) void block_sparse_attn_kernel(const AttnPar
     __builtin_amdgcn_s_waitcnt(0x0F70);   // this wave's share of block it+1's tiles has landed in LDS
     __syncthreads();   // block it+1's tiles are complete; the votes are visible; ring slot of block it-1 is free
     if (it + 2 < nv) {
-      blk_ld += lut_row[it + 2];
+      blk_ld = __builtin_amdgcn_readfirstlane(blk_ld + lut_row[it + 2]);
       const int b2 = buf == 0 ? 2 : buf - 1;   // (it+2) % 3
       SPG_LOAD_TILES(blk_ld, b2);
     }
