@@ -10,7 +10,8 @@ import os
 import torch
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "libspargeattn_amd.so")
+# SPARGEATTN_AMD_LIB lets a developer point at another build of the same library (A/B comparisons)
+LIB_PATH = os.environ.get("SPARGEATTN_AMD_LIB", os.path.join(_HERE, "libspargeattn_amd.so"))
 
 SPG_OK, SPG_ERR_INVALID, SPG_ERR_UNSUPPORTED, SPG_ERR_HIP = 0, 1, 2, 3
 SPG_F16, SPG_BF16 = 0, 1

@@ -67,9 +67,11 @@ __global__ __launch_bounds__(256, 3) void block_sparse_attn_kernel(const AttnPar
   constexpr int CPR = D / 16;       // 16-byte chunks per K row
   constexpr int WL = D / 64;        // global_load_lds instructions per wave per tile (TILE / 1024 / 4)
   constexpr int NBUF = 3;
-  __shared__ __align__(1024) unsigned char sK[NBUF][TILE];
-  __shared__ __align__(1024) unsigned char sV[NBUF][TILE];
+  // LDS: K ring [NBUF][TILE] | V^T ring [NBUF][TILE] | votes
+  __shared__ __align__(1024) unsigned char smem[2 * NBUF * TILE];
   __shared__ int sVote[2][4];
+  unsigned char *const sKr = smem;
+  unsigned char *const sVr = smem + NBUF * TILE;
 
   // ---- workgroup -> (batch*head, q block): one XCD per head at a time, heavy (late) rows first ----------
   const int w = blockIdx.x;
@@ -96,48 +98,69 @@ __global__ __launch_bounds__(256, 3) void block_sparse_attn_kernel(const AttnPar
 
   const int8_t *kbase = p.k8 + (size_t)bh * N * D;
   const uint8_t *vbase = p.v8 + (size_t)bh * p.nk * (size_t)TILE;
-  const float *kscale = p.k_scale + (size_t)bh * p.nk;
-  const float qs = p.q_scale[(size_t)bh * p.nq + qb];
+  // LUT and K scales are read through the constant address space: uniform addresses become scalar loads (SMEM),
+  // which never touch the vector-memory counter the tile ring is synchronised with.
+  typedef const __attribute__((address_space(4))) int32_t *c_i32_t;
+  typedef const __attribute__((address_space(4))) float *c_f32_t;
+  const c_i32_t lutc = (c_i32_t)(p.lut + ((size_t)bh * p.nq + qb) * p.nk);
+  const c_f32_t kscale = (c_f32_t)(p.k_scale + (size_t)bh * p.nk);
+  const float qs = ((c_f32_t)p.q_scale)[(size_t)bh * p.nq + qb];
   const float c = p.sm_scale_log2;
-  const float thr = p.pvthr[head];
+  const float thr = ((c_f32_t)p.pvthr)[head];
 
   // ---- tile loader: wave w copies LDS bytes [1024*(WL*w+u), +1024) of each tile, lane l the 16-byte chunk l ----
   // K: LDS chunk position pos <-> (row = pos / CPR, slot = pos % CPR) holds global chunk slot ^ k_swz(row).
-  // A tile's global address is (uniform base of the block) + (per-lane 32-bit offset): no per-load VALU work.
-  uint32_t k_lane[WL], v_lane[WL];
-#pragma unroll
-  for (int u = 0; u < WL; u++) {
-    const int pos = (WL * wave + u) * 64 + lane;
-    k_lane[u] = (uint32_t)((pos / CPR) * D + ((pos % CPR) ^ k_swz<D>(pos / CPR)) * 16);
-    v_lane[u] = (uint32_t)pos * 16u;
-  }
+  // A tile's global address is (uniform base of the block) + (per-lane 32-bit offset) + u*1024, and the same
+  // u*1024 is the LDS offset: it rides in the instruction's immediate (applied to both addresses).
+  // (the two per-lane offsets are recomputed from the thread id where they are used: cheaper than keeping them
+  //  in registers across the loop, where the register file is the scarce resource)
+#define SPG_LANE_OFFSETS()                                                                                    \
+  int tid_ = threadIdx.x;                                                                                     \
+  asm volatile("" : "+v"(tid_));                                                                              \
+  const int pos0 = WL * (tid_ >> 6) * 64 + (tid_ & 63);                                                       \
+  const uint32_t k_lane = (uint32_t)((pos0 / CPR) * D + ((pos0 % CPR) ^ k_swz<D>(pos0 / CPR)) * 16);          \
+  const uint32_t v_lane = (uint32_t)pos0 * 16u;
   const int last_partial_blk = (N % 64) ? p.nk - 1 : -1;   // the only block with rows beyond N
   typedef __attribute__((address_space(3))) void *lds_ptr_t;
   typedef const __attribute__((address_space(1))) void *glb_ptr_t;
-#define SPG_LOAD_TILES(BLK, BUF)                                                                              \
+#define SPG_LOAD_TILES(BLK, BUFOFF)                                                                           \
   {                                                                                                           \
+    SPG_LANE_OFFSETS()                                                                                        \
     const int8_t *kb_ = kbase + (size_t)(BLK) * TILE;                                                         \
     const uint8_t *vb_ = vbase + (size_t)(BLK) * TILE;                                                        \
-    const int rows_ok_ = N - (BLK) * 64; /* >= 64 except in the partial last block */                         \
-    _Pragma("unroll") for (int u = 0; u < WL; u++) {                                                          \
-      uint32_t ko_ = k_lane[u];                                                                               \
-      if ((BLK) == last_partial_blk) {                                                                        \
-        /* rows beyond N are clamped to row N-1: their scores are masked, their V rows are zero */            \
-        const int pos = (WL * wave + u) * 64 + lane;                                                          \
-        const int row_ = min(pos / CPR, rows_ok_ - 1);                                                        \
-        ko_ = (uint32_t)(row_ * D + ((pos % CPR) ^ k_swz<D>(pos / CPR)) * 16);                                \
+    unsigned char *lk_ = sKr + (BUFOFF) + WL * wave * 1024;                                                   \
+    unsigned char *lv_ = sVr + (BUFOFF) + WL * wave * 1024;                                                   \
+    if ((BLK) != last_partial_blk) {                                                                          \
+      __builtin_amdgcn_global_load_lds((glb_ptr_t)(kb_ + k_lane), (lds_ptr_t)lk_, 16, 0, 0);                  \
+      __builtin_amdgcn_global_load_lds((glb_ptr_t)(vb_ + v_lane), (lds_ptr_t)lv_, 16, 0, 0);                  \
+      if constexpr (WL == 2) {                                                                                \
+        __builtin_amdgcn_global_load_lds((glb_ptr_t)(kb_ + k_lane), (lds_ptr_t)lk_, 16, 1024, 0);             \
+        __builtin_amdgcn_global_load_lds((glb_ptr_t)(vb_ + v_lane), (lds_ptr_t)lv_, 16, 1024, 0);             \
       }                                                                                                       \
-      __builtin_amdgcn_global_load_lds((glb_ptr_t)(kb_ + ko_), (lds_ptr_t)(sK[BUF] + (WL * wave + u) * 1024), \
-                                       16, 0, 0);                                                             \
-      __builtin_amdgcn_global_load_lds((glb_ptr_t)(vb_ + v_lane[u]),                                          \
-                                       (lds_ptr_t)(sV[BUF] + (WL * wave + u) * 1024), 16, 0, 0);              \
+    } else {                                                                                                  \
+      /* rows beyond N are clamped to row N-1: their scores are masked, their V rows are zero */              \
+      const int rows_ok_ = N - (BLK) * 64;                                                                    \
+      _Pragma("unroll") for (int u = 0; u < WL; u++) {                                                        \
+        const int pos = pos0 + u * 64;                                                                        \
+        const int row_ = min(pos / CPR, rows_ok_ - 1);                                                        \
+        const uint32_t ko_ = (uint32_t)(row_ * D + ((pos % CPR) ^ k_swz<D>(pos / CPR)) * 16);                 \
+        __builtin_amdgcn_global_load_lds((glb_ptr_t)(kb_ + ko_), (lds_ptr_t)(lk_ + u * 1024), 16, 0, 0);      \
+        __builtin_amdgcn_global_load_lds((glb_ptr_t)(vb_ + v_lane + u * 1024), (lds_ptr_t)(lv_ + u * 1024), 16, 0, 0); \
+      }                                                                                                       \
     }                                                                                                         \
   }
 
-  // MFMA row i of key tile kt carries key 32*((i>>2)&1) + 16*kt + 4*(i>>3) + (i&3)
+  // MFMA row i of key tile kt carries key 32*((i>>2)&1) + 16*kt + 4*(i>>3) + (i&3); rows krow0 and krow0+16 have
+  // the same swizzle, so tile 1's operand sits 16 rows (16*D bytes) after tile 0's.
   const int krow0 = 32 * ((r >> 2) & 1) + 4 * (r >> 3) + (r & 3);
-  const int ksw0 = k_swz<D>(krow0), ksw1 = k_swz<D>(krow0 + 16);
-  const int vsw = v_swz(r);     // v_swz(32*dt + r) does not depend on dt
+  const int ksw = k_swz<D>(krow0);
+  // K operand of k-step ks (tile 0): chunk (2ks+hh) ^ ksw = ((2ks) ^ (ksw & 6)) | ((hh ^ ksw) & 1), i.e. the LDS
+  // byte offset is k_rd_base + ((32*ks) ^ k_rd_x): one xor-add per read, two registers.
+  const uint32_t k_rd_base = (uint32_t)(krow0 * D + ((hh ^ ksw) & 1) * 16);
+  const uint32_t k_rd_x = (uint32_t)((ksw & 6) * 16);
+  const int vsw = v_swz(r);                // v_swz(32*dt + r) does not depend on dt
+  // V^T operand: key chunks 2hh and 2hh+1 of channel row r (+32*dt); the two swizzled slots differ in bit 4 only
+  const uint32_t v_rd_lo = (uint32_t)(r * 64 + (((2 * hh) ^ vsw) * 16));
 
   float m = SPG_NEG_BIG;
   float dsum = hh == 0 ? 1.0f : 0.0f;     // the two half-lanes of a query share d = 1.0 (sm89.cuh:172)
@@ -148,15 +171,16 @@ __global__ __launch_bounds__(256, 3) void block_sparse_attn_kernel(const AttnPar
     for (int e = 0; e < 16; e++) O[dt][e] = 0.f;
   int cnt = 0;
 
-  int blk = __builtin_amdgcn_readfirstlane(lut_row[0]);   // block computed in the current iteration
-  int blk_ld = blk;                                         // last block whose loads were issued
+  // block ids: blk = block of iteration it, blk1 = it+1, blk2 = it+2 (tiles in flight); d3 = LUT delta of it+3.
+  // K scales are fetched one iteration ahead as well.
+  int blk = lutc[0];
+  int blk1 = blk + (nv > 1 ? lutc[1] : 0);
+  int blk2 = blk1 + (nv > 2 ? lutc[2] : 0);
+  int d3 = nv > 3 ? lutc[3] : 0;
+  float ksc = kscale[blk], ksc1 = kscale[blk1];
   SPG_LOAD_TILES(blk, 0);
-  if (nv > 1) {
-    blk_ld = __builtin_amdgcn_readfirstlane(blk + lut_row[1]);
-    SPG_LOAD_TILES(blk_ld, 1);
-  }
-  int blk_n1 = blk_ld;         // block of iteration it+1
-  int buf = 0;
+  if (nv > 1) SPG_LOAD_TILES(blk1, TILE);
+  uint32_t bufoff = 0;                     // LDS ring offset of block it
 
 #pragma unroll 1
   for (int it = 0; it < nv; it++) {
@@ -164,21 +188,25 @@ __global__ __launch_bounds__(256, 3) void block_sparse_attn_kernel(const AttnPar
       __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0)
       __syncthreads();
     }
+    // scalar prefetches for later iterations (SMEM)
+    const float ksc2 = kscale[blk2];
+    const int d4 = it + 4 < nv ? lutc[it + 4] : 0;
+
     // ---- S^T = K . Q^T ---------------------------------------------------------------------------------
     v16i S0, S1;
 #pragma unroll
     for (int e = 0; e < 16; e++) { S0[e] = 0; S1[e] = 0; }
+    const unsigned char *kt = sKr + bufoff;
 #pragma unroll
     for (int ks = 0; ks < KS; ks++) {
-      const int ch = 2 * ks + hh;
-      const v4i a0 = *(const v4i *)(sK[buf] + krow0 * D + ((ch ^ ksw0) * 16));
-      const v4i a1 = *(const v4i *)(sK[buf] + (krow0 + 16) * D + ((ch ^ ksw1) * 16));
+      const uint32_t ko = k_rd_base + ((uint32_t)(32 * ks) ^ k_rd_x);
+      const v4i a0 = *(const v4i *)(kt + ko);
+      const v4i a1 = *(const v4i *)(kt + ko + 16 * D);
       S0 = __builtin_amdgcn_mfma_i32_32x32x32_i8(a0, qreg[ks], S0, 0, 0, 0);
       S1 = __builtin_amdgcn_mfma_i32_32x32x32_i8(a1, qreg[ks], S1, 0, 0, 0);
     }
 
-    const int cur = blk;
-    const float dq = qs * kscale[cur];
+    const float dq = qs * ksc;
     const bool tail = it >= nv - 2;   // last two blocks: masks, no PV skip (sm89.cuh:467-648)
     float x[32];
     float a, fm;
@@ -193,8 +221,8 @@ __global__ __launch_bounds__(256, 3) void block_sparse_attn_kernel(const AttnPar
       a = c * dq;
       fm = (float)imax * a;
     } else {
-      // slot e of this lane is key 64*cur + 32*hh + e; keys beyond `lim` are masked
-      const int key0 = cur * 64 + 32 * hh;
+      // slot e of this lane is key 64*blk + 32*hh + e; keys beyond `lim` are masked
+      const int key0 = blk * 64 + 32 * hh;
       int lim = 0x7fffffff;
       if (p.is_causal) lim = q_row - key0;                       // key > query (attn_utils.cuh:334-361)
       if (it == nv - 1) lim = min(lim, N - 1 - key0);            // key >= kv_len (attn_utils.cuh:363-389)
@@ -222,9 +250,8 @@ __global__ __launch_bounds__(256, 3) void block_sparse_attn_kernel(const AttnPar
     __builtin_amdgcn_s_waitcnt(0x0F70);   // this wave's share of block it+1's tiles has landed in LDS
     __syncthreads();   // block it+1's tiles are complete; the votes are visible; ring slot of block it-1 is free
     if (it + 2 < nv) {
-      blk_ld = __builtin_amdgcn_readfirstlane(blk_ld + lut_row[it + 2]);
-      const int b2 = buf == 0 ? 2 : buf - 1;   // (it+2) % 3
-      SPG_LOAD_TILES(blk_ld, b2);
+      const uint32_t b2 = bufoff == 0 ? 2 * TILE : bufoff - TILE;   // slot (it+2) % 3
+      SPG_LOAD_TILES(blk2, b2);
     }
     bool compute = true;
     if (!tail)         // workgroup-uniform (PVThresholdMode::kPerBlock, sm89.cuh:318-353)
@@ -249,25 +276,28 @@ __global__ __launch_bounds__(256, 3) void block_sparse_attn_kernel(const AttnPar
       v8i pb;
 #pragma unroll
       for (int u = 0; u < 8; u++) {
-        int wv = __builtin_amdgcn_cvt_pk_fp8_f32(x[4 * u], x[4 * u + 1], 0, false);
+        // both halves of the destination are written: the initial content is irrelevant, so the register of
+        // x[4u] is reused instead of a zeroed one
+        int wv = __builtin_amdgcn_cvt_pk_fp8_f32(x[4 * u], x[4 * u + 1], __builtin_bit_cast(int, x[4 * u]), false);
         wv = __builtin_amdgcn_cvt_pk_fp8_f32(x[4 * u + 2], x[4 * u + 3], wv, true);
         pb[u] = wv;
       }
+      const unsigned char *vt = sVr + bufoff;
 #pragma unroll
       for (int dt = 0; dt < NDT; dt++) {
-        const unsigned char *vrow = sV[buf] + (32 * dt + r) * 64;
-        const v4i lo = *(const v4i *)(vrow + (((2 * hh) ^ vsw) * 16));
-        const v4i hi = *(const v4i *)(vrow + (((2 * hh + 1) ^ vsw) * 16));
+        const v4i lo = *(const v4i *)(vt + v_rd_lo + dt * 2048);
+        const v4i hi = *(const v4i *)(vt + (v_rd_lo ^ 16u) + dt * 2048);
         const v8i av = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
         O[dt] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(av, pb, O[dt], 0, 0, 0, 0, 0, 0);
       }
     }
-    // advance: block of iteration it+1, then the one after
-    blk = blk_n1;
-    blk_n1 = blk_ld;
-    buf = buf == NBUF - 1 ? 0 : buf + 1;
+    // advance the block pipeline and the ring
+    blk = blk1; blk1 = blk2; blk2 = blk2 + d3; d3 = d4;
+    ksc = ksc1; ksc1 = ksc2;
+    bufoff = bufoff == 2 * TILE ? 0 : bufoff + TILE;
   }
 #undef SPG_LOAD_TILES
+#undef SPG_LANE_OFFSETS
 
   if (p.pv_count != nullptr && tid == 0) p.pv_count[(size_t)bh * p.nq + qb] = cnt;
 
