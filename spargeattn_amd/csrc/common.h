@@ -100,6 +100,25 @@ __device__ __forceinline__ float half_swap_sum_f32(float v) {
   return lo + hi;
 }
 
+// Sum over aligned groups of G lanes (G in {2,4,8,16}) with DPP lane permutes (VALU rate, no LDS traffic).
+// Steps: xor 1, xor 2 (quad permutes), then half-row mirror and row mirror, which pair a group with its sibling
+// once the values are uniform inside the group.  Every lane of the group ends with the same total.
+template <int CTRL>
+__device__ __forceinline__ double dpp_f64(double v) {
+  const uint64_t u = __builtin_bit_cast(uint64_t, v);
+  const int lo = __builtin_amdgcn_update_dpp(0, (int)(uint32_t)u, CTRL, 0xf, 0xf, true);
+  const int hi = __builtin_amdgcn_update_dpp(0, (int)(uint32_t)(u >> 32), CTRL, 0xf, 0xf, true);
+  return __builtin_bit_cast(double, ((uint64_t)(uint32_t)hi << 32) | (uint32_t)lo);
+}
+template <int G>
+__device__ __forceinline__ double group_sum_f64(double v) {
+  if constexpr (G >= 2) v += dpp_f64<0xB1>(v);    // quad_perm [1,0,3,2]
+  if constexpr (G >= 4) v += dpp_f64<0x4E>(v);    // quad_perm [2,3,0,1]
+  if constexpr (G >= 8) v += dpp_f64<0x141>(v);   // row_half_mirror
+  if constexpr (G >= 16) v += dpp_f64<0x140>(v);  // row_mirror
+  return v;
+}
+
 __device__ __forceinline__ float wave_max_f32(float v) {
 #pragma unroll
   for (int o = 32; o >= 1; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, SPG_WAVE));

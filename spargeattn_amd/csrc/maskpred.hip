@@ -66,6 +66,23 @@ __global__ void km_final_kernel(const double *__restrict__ part, uint16_t *__res
 // =============================================================================================
 // pool + sim + INT8 quantisation.  One workgroup per (block, b*h).
 // =============================================================================================
+// IEEE binary32 quotient a/b through a refined reciprocal r ~ 1/b shared by many numerators: the operation
+// sequence of the hardware's correctly rounded division (reciprocal + one Newton step, then two residual
+// corrections of the quotient) without its operand scaling, valid while b stays in [2^-60, 2^60].
+__device__ __forceinline__ float refined_rcp(float b) {
+  const float r0 = __builtin_amdgcn_rcpf(b);
+  const float e = __builtin_fmaf(-b, r0, 1.0f);
+  return __builtin_fmaf(e, r0, r0);
+}
+__device__ __forceinline__ float div_by(float a, float b, float r) {
+  float q = a * r;
+  float e = __builtin_fmaf(-b, q, a);
+  q = __builtin_fmaf(e, r, q);
+  e = __builtin_fmaf(-b, q, a);
+  return __builtin_fmaf(e, r, q);
+}
+__device__ __forceinline__ bool rcp_safe(float b) { return b >= 0x1p-60f && b <= 0x1p60f; }
+
 template <int BS, int D, int DT, bool HAS_MEAN, bool WITH_POOL>
 __global__ __launch_bounds__(256) void pool_sim_quant_kernel(const uint16_t *__restrict__ x,
                                                              const uint16_t *__restrict__ km,
@@ -105,8 +122,10 @@ __global__ __launch_bounds__(256) void pool_sim_quant_kernel(const uint16_t *__r
     for (int e = 0; e < 8; e++) {
       float f = elem_to_f32<DT>((uint16_t)((e & 1) ? (w[e >> 1] >> 16) : (w[e >> 1] & 0xffffu)));
       if constexpr (HAS_MEAN) {
-        // (k - km) rounded once to the input dtype; masked rows stay zero (utils.py:184-188)
-        if (ok) f = elem_to_f32<DT>(f64_to_elem<DT>((double)f - (double)kmf[e]));
+        // (k - km) rounded once to the input dtype (utils.py:184-188).  The binary32 difference of two 16-bit
+        // floats is either exact or nowhere near a rounding tie of the 16-bit format, so rounding it to nearest
+        // even equals rounding the exact difference.  Masked rows stay zero.
+        if (ok) f = elem_to_f32<DT>(f32_to_elem<DT>(f - kmf[e]));
       }
       xf[p][e] = f;
       amax = fmaxf(amax, fabsf(f));
@@ -120,48 +139,56 @@ __global__ __launch_bounds__(256) void pool_sim_quant_kernel(const uint16_t *__r
 
   if constexpr (WITH_POOL) {
     __shared__ double s_col[RPP][D];
-    __shared__ long long s_xi[RPP][D];
-    double colsum[8];
-    long long colxi[8];
+    __shared__ double s_xh[RPP][D];
+    double colsum[8], colxh[8];
 #pragma unroll
-    for (int e = 0; e < 8; e++) { colsum[e] = 0.0; colxi[e] = 0; }
-    int bad = 0;
+    for (int e = 0; e < 8; e++) { colsum[e] = 0.0; colxh[e] = 0.0; }
 #pragma unroll
     for (int p = 0; p < NP; p++) {
       double ss = 0.0;
 #pragma unroll
       for (int e = 0; e < 8; e++) {
         const double xd = (double)xf[p][e];
-        ss += xd * xd;
+        ss = __builtin_fma(xd, xd, ss);             // squares and their sum are exact in binary64
         colsum[e] += xd;
       }
-#pragma unroll
-      for (int o = TPR / 2; o >= 1; o >>= 1) ss += shfl_xor_f64(ss, o);
+      ss = group_sum_f64<TPR>(ss);                 // the TPR lanes of this row
       const float norm = sqrtf((float)ss);
+      if (rcp_safe(norm)) {
+        const float rn = refined_rcp(norm);
 #pragma unroll
-      for (int e = 0; e < 8; e++) {
-        const float xh = xf[p][e] / norm;          // 0/0 -> NaN for all-zero (masked) rows
-        const _Float16 h = (_Float16)xh;
-        const float hf = (float)h;
-        if (__builtin_isfinite(hf)) colxi[e] += (long long)(int)(hf * 16777216.0f);  // exact: fp16 = int * 2^-24
-        else bad = 1;
+        for (int e = 0; e < 8; e++) {
+          const _Float16 h = (_Float16)div_by(xf[p][e], norm, rn);
+          colxh[e] += (double)(float)h;             // fp16 values: integer multiples of 2^-24, sums are exact
+        }
+      } else {
+#pragma unroll
+        for (int e = 0; e < 8; e++) {
+          const _Float16 h = (_Float16)(xf[p][e] / norm);   // 0/0 -> NaN for all-zero (masked) rows
+          colxh[e] += (double)(float)h;
+        }
       }
     }
 #pragma unroll
-    for (int e = 0; e < 8; e++) { s_col[r][c * 8 + e] = colsum[e]; s_xi[r][c * 8 + e] = colxi[e]; }
-    const int any_bad = __syncthreads_or(bad);
+    for (int e = 0; e < 8; e++) { s_col[r][c * 8 + e] = colsum[e]; s_xh[r][c * 8 + e] = colxh[e]; }
+    __syncthreads();
     long long g = 0;
+    int bad = 0;
     if (tid < D) {
-      double s = 0.0;
-      long long sx = 0;
-      for (int i = 0; i < RPP; i++) { s += s_col[i][tid]; sx += s_xi[i][tid]; }
+      double s = 0.0, sx = 0.0;
+      for (int i = 0; i < RPP; i++) { s += s_col[i][tid]; sx += s_xh[i][tid]; }
       pool[((size_t)bh * nb + blk) * D + tid] = f64_to_elem<DT>(s / (double)rows_valid);
-      g = sx * sx;
+      if (__builtin_isfinite(sx)) {
+        const long long si = (long long)(sx * 16777216.0);   // exact integer
+        g = si * si;
+      } else {
+        bad = 1;                                    // a NaN/inf x_hat anywhere in the column
+      }
     }
 #pragma unroll
     for (int o = 32; o >= 1; o >>= 1) g += shfl_xor_i64(g, o);
     if ((tid & 63) == 0) s_wg[tid >> 6] = g;
-    __syncthreads();
+    const int any_bad = __syncthreads_or(bad);
     if (tid == 0) {
       const long long gt = s_wg[0] + s_wg[1] + s_wg[2] + s_wg[3];   // = sum(gram) * 2^48, exact
       const double thr = (double)simthr[bh % H] * (double)(rows_valid * rows_valid) * 281474976710656.0;
@@ -174,20 +201,28 @@ __global__ __launch_bounds__(256) void pool_sim_quant_kernel(const uint16_t *__r
   amax = fmaxf(fmaxf(s_wmax[0], s_wmax[1]), fmaxf(s_wmax[2], s_wmax[3]));
   const float s = amax / 127.0f + 1e-7f;
   int8_t *qb = xq + ((size_t)bh * N + row_base) * D + c * 8;
+  auto quantise = [&](auto divide) {
 #pragma unroll
-  for (int p = 0; p < NP; p++) {
-    const int row = r + p * RPP;
-    if (row < rows_valid) {
-      uint32_t pk[2] = {0, 0};
+    for (int p = 0; p < NP; p++) {
+      const int row = r + p * RPP;
+      if (row < rows_valid) {
+        uint32_t pk[2] = {0, 0};
 #pragma unroll
-      for (int e = 0; e < 8; e++) {
-        float y = xf[p][e] / s;
-        y = y + (y >= 0.f ? 0.5f : -0.5f);
-        const int q = (int)y;   // truncation toward zero
-        pk[e >> 2] |= ((uint32_t)q & 0xffu) << (8 * (e & 3));
+        for (int e = 0; e < 8; e++) {
+          float y = divide(xf[p][e]);
+          y = y + (y >= 0.f ? 0.5f : -0.5f);
+          const int q = (int)y;   // truncation toward zero
+          pk[e >> 2] |= ((uint32_t)q & 0xffu) << (8 * (e & 3));
+        }
+        *(uint2 *)(qb + (size_t)row * D) = make_uint2(pk[0], pk[1]);
       }
-      *(uint2 *)(qb + (size_t)row * D) = make_uint2(pk[0], pk[1]);
     }
+  };
+  if (rcp_safe(s)) {                     // workgroup-uniform
+    const float rs = refined_rcp(s);
+    quantise([&](float v) { return div_by(v, s, rs); });
+  } else {
+    quantise([&](float v) { return v / s; });
   }
   if (tid == 0) scale[(size_t)bh * nb + blk] = s;
 }

@@ -82,3 +82,32 @@ def test_e4m3_saturates_and_nan():
     got = R.f32_to_e4m3fn(x)
     assert list(got[:6]) == [0x7E, 0x7E, 0x7E, 0x7E, 0x7E, 0xFE]
     assert got[6] & 0x7F == 0x7F
+
+
+def test_fp32_subtraction_then_rne_equals_single_rounding():
+    """Lemma the GPU smoothing step relies on: for a, b in T, RN_T(RN_f32(a - b)) == RN_T(a - b).
+
+    Checked on random pairs with every exponent gap from 0 to 30 (where the binary32 difference stops being exact)
+    and on values next to powers of two, for both 16-bit formats."""
+    rng = np.random.default_rng(11)
+    for tag in (R.BF16, R.FP16):
+        pats = np.arange(0x0080 if tag == R.BF16 else 0x0001, 0x7F80 if tag == R.BF16 else 0x7C00, dtype=np.uint16)
+        vals = R.from_bits16(pats, tag).astype(np.float64)
+        vals = vals[(vals > 1e-30) & (vals < 1e30)]
+        a = rng.choice(vals, 400000) * rng.choice([-1.0, 1.0], 400000)
+        gaps = rng.integers(0, 31, 400000)
+        b = rng.choice(vals, 400000)
+        b = b * 2.0 ** (np.floor(np.log2(np.abs(a))) - gaps - np.floor(np.log2(b)))      # force the exponent gap
+        b = R.round_to(b, tag).astype(np.float64) * rng.choice([-1.0, 1.0], 400000)
+        keep = np.isfinite(b) & (b != 0)
+        a, b = a[keep], b[keep]
+        exact = R.round_to(a - b, tag)
+        via32 = R.round_to((a.astype(np.float32) - b.astype(np.float32)).astype(np.float64), tag)
+        assert np.array_equal(exact, via32), tag
+        # neighbours of powers of two (where the spacing halves)
+        p2 = 2.0 ** rng.integers(-10, 10, 100000)
+        ulp = p2 * (2.0 ** -7 if tag == R.BF16 else 2.0 ** -10)
+        a2 = R.round_to(p2 + rng.integers(-2, 3, 100000) * ulp / 2, tag).astype(np.float64)
+        b2 = R.round_to(p2 * 2.0 ** -rng.integers(8, 26, 100000), tag).astype(np.float64)
+        assert np.array_equal(R.round_to(a2 - b2, tag),
+                              R.round_to((a2.astype(np.float32) - b2.astype(np.float32)).astype(np.float64), tag))
