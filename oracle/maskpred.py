@@ -208,19 +208,16 @@ def pool_sim_quant(x, km, bs, simthreshd1, dtype, with_pool=True):
 def pooled_scores(pool_q, pool_k, dtype):
     """(pooledQ @ pooledK^T) -> T, then * fp32(D**-0.5) -> T (utils.py:388).
 
-    Fixed order of the dot product: D/8 lanes, lane g adds the products of d = 8g .. 8g+7 in order, the partial
-    sums are combined by an xor-butterfly.  (Products of two T values are exact in binary64.)
+    Fixed order of the dot product: binary64 accumulation over d = 0, 1, ..., D-1.  (Products of two T values are
+    exact in binary64.)
     """
     pq = np.asarray(pool_q, dtype=F64)
     pk = np.asarray(pool_k, dtype=F64)
     d = pq.shape[-1]
-    g = d // 8
-    pq = pq.reshape(pq.shape[:-1] + (g, 8))
-    pk = pk.reshape(pk.shape[:-1] + (g, 8))
-    acc = np.zeros(pq.shape[:-2] + (pk.shape[-3], g), dtype=F64)          # (..., nq, nk, g)
-    for e in range(8):
-        acc = acc + pq[..., :, None, :, e] * pk[..., None, :, :, e]
-    s1 = round_to(_butterfly(acc, g), dtype)
+    acc = np.zeros(pq.shape[:-1] + (pk.shape[-2],), dtype=F64)
+    for i in range(d):
+        acc = acc + pq[..., :, i, None] * pk[..., None, :, i]
+    s1 = round_to(acc, dtype)
     return round_to(s1.astype(F64) * F64(F32(d ** -0.5)), dtype)
 
 

@@ -291,160 +291,179 @@ __device__ __forceinline__ void emit_lut(FlagFn flag, int nk, int nkp, int32_t *
 }
 
 // =============================================================================================
-// block_select: one workgroup per (q block row, b*h).
-// dynamic LDS: 12 * nkp bytes (nkp = power of two >= max(nk, 256)).
+// block_select: one workgroup per (R consecutive q block rows, b*h).
+// Phase 1 computes the R x nk pooled scores with every pooled-K row read ONCE for the R rows (one lane per
+// column, binary64 accumulation in the fixed order d = 0..D-1); phase 2 handles the rows one after the other:
+// softmax, stable descending sort, top-k / CDF count, block-map row, delta LUT.
+// dynamic LDS: R*D*8 (pooled Q as doubles) + R*nkp*4 (scores) + 12*nkp (per-row work area).
 // =============================================================================================
-template <int D, int DT>
-__global__ __launch_bounds__(256, 4) void block_select_kernel(
+template <int D, int DT, int R>
+__global__ __launch_bounds__(256) void block_select_kernel(
     const uint16_t *__restrict__ pool_q, const uint8_t *__restrict__ sim_q, const uint16_t *__restrict__ pool_k,
     const uint8_t *__restrict__ sim_k, const float *__restrict__ topk, const float *__restrict__ cdfthr, int is_causal,
     int sink, int32_t *__restrict__ lut, int32_t *__restrict__ valid, uint8_t *__restrict__ bmap, int H, int nq, int nk,
     int nkp) {
   extern __shared__ __align__(16) unsigned char smem[];
-  double *e_buf = (double *)smem;                    // [nkp] exp values        (phase 1)
-  uint32_t *skey = (uint32_t *)smem;                 // [nkp] sorted keys       (phase 2, aliases e_buf)
-  int32_t *s_idx = (int32_t *)(smem + 4 * (size_t)nkp);  // [nkp] compact indices (phase 3, aliases e_buf)
-  uint32_t *okey = (uint32_t *)(smem + 8 * (size_t)nkp); // [nkp] scores, then keys in column order
-  __shared__ float s_pq[D];
+  double *s_pq = (double *)smem;                                   // [R][D]
+  float *s_scores = (float *)(smem + (size_t)R * D * 8);           // [R][nkp]
+  unsigned char *work = smem + (size_t)R * D * 8 + (size_t)R * nkp * 4;
+  double *e_buf = (double *)work;                      // [nkp] exp values        (step 1)
+  uint32_t *skey = (uint32_t *)work;                   // [nkp] sorted keys       (step 2, aliases e_buf)
+  int32_t *s_idx = (int32_t *)(work + 4 * (size_t)nkp);    // [nkp] compact indices (step 3, aliases e_buf)
+  uint32_t *okey = (uint32_t *)(work + 8 * (size_t)nkp);   // [nkp] keys in column order
   __shared__ float s_wmax[4];
   __shared__ double s_wsum[4];
   __shared__ double s_tsum[256];
   __shared__ int s_tmp[256];
   __shared__ int s_n;
 
-  const int i = blockIdx.x, bh = blockIdx.y, h = bh % H, tid = threadIdx.x;
-  if (tid < D) s_pq[tid] = elem_to_f32<DT>(pool_q[((size_t)bh * nq + i) * D + tid]);
+  const int i0 = blockIdx.x * R, bh = blockIdx.y, h = bh % H, tid = threadIdx.x;
+  const int rows = min(R, nq - i0);
+  for (int t = tid; t < R * D; t += 256) {
+    const int row = t / D;
+    s_pq[t] = row < rows ? (double)elem_to_f32<DT>(pool_q[((size_t)bh * nq + i0 + row) * D + (t % D)]) : 0.0;
+  }
   __syncthreads();
 
   const float sm_scale = (D == 64) ? 0.125f : 0.088388347648318447f;  // fp32(D^-0.5)
-  const int causal_lim = is_causal ? min(nk, 2 * (i + 1)) : nk;
   const uint16_t *pk_base = pool_k + (size_t)bh * nk * D;
   const uint8_t *simk = sim_k + (size_t)bh * nk;
-  float *s_score = (float *)okey;
 
-  // ---- scores: G = D/8 lanes share one column (one coalesced 16-byte load each); a lane adds its 8 products
-  //      in order, the G partial sums are combined by an xor butterfly (offsets G/2 .. 1).  Two roundings to the
-  //      input dtype, then the masks.
-  constexpr int G = D / 8;
-  const int g = tid % G, cg = tid / G;
-  float pqv[8];
+  // ---- phase 1: scores.  Products of two 16-bit floats are exact in binary64, so fma == multiply-then-add. ----
+  for (int j = tid; j < nk; j += 256) {
+    double acc[R];
 #pragma unroll
-  for (int e = 0; e < 8; e++) pqv[e] = s_pq[g * 8 + e];
-  float lmax = -INFINITY;
-  for (int j0 = 0; j0 < nk; j0 += 256 / G) {
-    const int j = j0 + cg;
-    double acc = 0.0;
-    if (j < nk) {
-      const uint4 v = *(const uint4 *)(pk_base + (size_t)j * D + g * 8);
+    for (int row = 0; row < R; row++) acc[row] = 0.0;
+    const uint4 *krow = (const uint4 *)(pk_base + (size_t)j * D);
+#pragma unroll 2
+    for (int cch = 0; cch < D / 8; cch++) {
+      const uint4 v = krow[cch];
       const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+      double kd[8];
 #pragma unroll
-      for (int e = 0; e < 8; e++) {
-        const float kf = elem_to_f32<DT>((uint16_t)((e & 1) ? (w[e >> 1] >> 16) : (w[e >> 1] & 0xffffu)));
-        acc = acc + (double)pqv[e] * (double)kf;   // product exact in binary64
+      for (int e = 0; e < 8; e++)
+        kd[e] = (double)elem_to_f32<DT>((uint16_t)((e & 1) ? (w[e >> 1] >> 16) : (w[e >> 1] & 0xffffu)));
+#pragma unroll
+      for (int row = 0; row < R; row++) {
+        const double *q = s_pq + row * D + cch * 8;
+#pragma unroll
+        for (int e = 0; e < 8; e++) acc[row] = __builtin_fma(q[e], kd[e], acc[row]);
       }
     }
+    const bool dead_col = simk[j] == 0;
 #pragma unroll
-    for (int o = G / 2; o >= 1; o >>= 1) acc = acc + shfl_xor_f64(acc, o);
-    if (g == 0 && j < nk) {
-      const float s1 = elem_to_f32<DT>(f64_to_elem<DT>(acc));
+    for (int row = 0; row < R; row++) {
+      const float s1 = elem_to_f32<DT>(f64_to_elem<DT>(acc[row]));
       float s2 = elem_to_f32<DT>(f64_to_elem<DT>((double)s1 * (double)sm_scale));
-      if (!simk[j] || j >= causal_lim) s2 = -INFINITY;
-      s_score[j] = s2;
-      lmax = fmaxf(lmax, s2);
+      if (dead_col || (is_causal && j >= 2 * (i0 + row + 1))) s2 = -INFINITY;
+      s_scores[(size_t)row * nkp + j] = s2;
     }
   }
-  lmax = wave_max_f32(lmax);
-  if ((tid & 63) == 0) s_wmax[tid >> 6] = lmax;
   __syncthreads();
-  const float mx = fmaxf(fmaxf(s_wmax[0], s_wmax[1]), fmaxf(s_wmax[2], s_wmax[3]));
 
-  // ---- exp, then the fixed summation tree: lane l of ONE wavefront adds e[l], e[l+64], ... in order, followed
-  //      by an xor butterfly (32 .. 1) ------------------------------------------------------------------------
-  for (int j = tid; j < nk; j += 256) {
-    const float s2 = s_score[j];
-    e_buf[j] = (s2 == -INFINITY) ? 0.0 : cexp((double)s2 - (double)mx);
-  }
-  __syncthreads();
-  if (tid < 64) {
-    double part = 0.0;
-    for (int j = tid; j < nk; j += 64) part = part + e_buf[j];
+  // ---- phase 2: one row at a time ------------------------------------------------------------------------
+  for (int row = 0; row < rows; row++) {
+    const int i = i0 + row;
+    const int causal_lim = is_causal ? min(nk, 2 * (i + 1)) : nk;
+    const float *s_score = s_scores + (size_t)row * nkp;
+
+    float lmax = -INFINITY;
+    for (int j = tid; j < nk; j += 256) lmax = fmaxf(lmax, s_score[j]);
+    lmax = wave_max_f32(lmax);
+    if ((tid & 63) == 0) s_wmax[tid >> 6] = lmax;
+    __syncthreads();
+    const float mx = fmaxf(fmaxf(s_wmax[0], s_wmax[1]), fmaxf(s_wmax[2], s_wmax[3]));
+
+    // exp, then the fixed summation tree: lane l of ONE wavefront adds e[l], e[l+64], ... in order, followed by an
+    // xor butterfly (32 .. 1)
+    for (int j = tid; j < nk; j += 256) {
+      const float s2 = s_score[j];
+      e_buf[j] = (s2 == -INFINITY) ? 0.0 : cexp((double)s2 - (double)mx);
+    }
+    __syncthreads();
+    if (tid < 64) {
+      double part = 0.0;
+      for (int j = tid; j < nk; j += 64) part = part + e_buf[j];
 #pragma unroll
-    for (int o = 32; o >= 1; o >>= 1) part = part + shfl_xor_f64(part, o);
-    if (tid == 0) s_wsum[0] = part;
-  }
-  __syncthreads();
-  const double total = s_wsum[0];
+      for (int o = 32; o >= 1; o >>= 1) part = part + shfl_xor_f64(part, o);
+      if (tid == 0) s_wsum[0] = part;
+    }
+    __syncthreads();
+    const double total = s_wsum[0];
 
-  // ---- probabilities -> sortable keys (value bits, then lower index first) --------------------------
-  for (int j = tid; j < nk; j += 256) {
-    double p = e_buf[j] / total;
-    if (!__builtin_isfinite(p)) p = 0.0;
-    const uint32_t bits = f64_to_elem<DT>(p);
-    okey[j] = (bits << 16) | (0xffffu - (uint32_t)j);
-  }
-  __syncthreads();
-  for (int j = tid; j < nkp; j += 256) skey[j] = (j < nk) ? okey[j] : 0u;
-  __syncthreads();
+    // probabilities -> sortable keys (value bits, then lower index first)
+    for (int j = tid; j < nk; j += 256) {
+      double p = e_buf[j] / total;
+      if (!__builtin_isfinite(p)) p = 0.0;
+      const uint32_t bits = f64_to_elem<DT>(p);
+      okey[j] = (bits << 16) | (0xffffu - (uint32_t)j);
+    }
+    __syncthreads();
+    for (int j = tid; j < nkp; j += 256) skey[j] = (j < nk) ? okey[j] : 0u;
+    __syncthreads();
 
-  // ---- bitonic sort, descending ----------------------------------------------------------------------
-  for (int k = 2; k <= nkp; k <<= 1) {
-    for (int j = k >> 1; j > 0; j >>= 1) {
-      for (int t = tid; t < nkp / 2; t += 256) {
-        const int lo = ((t / j) * 2 * j) + (t % j);
-        const int hi = lo + j;
-        const bool desc = (lo & k) == 0;
-        const uint32_t a = skey[lo], b = skey[hi];
-        if ((a < b) == desc) { skey[lo] = b; skey[hi] = a; }
+    // bitonic sort, descending
+    for (int k = 2; k <= nkp; k <<= 1) {
+      for (int lj = __builtin_ctz(k) - 1; lj >= 0; lj--) {     // compare distance j = 2^lj
+        const int j = 1 << lj;
+        for (int t = tid; t < nkp / 2; t += 256) {
+          const int lo = ((t >> lj) << (lj + 1)) | (t & (j - 1));
+          const int hi = lo | j;
+          const bool desc = (lo & k) == 0;
+          const uint32_t a = skey[lo], b = skey[hi];
+          if ((a < b) == desc) { skey[lo] = b; skey[hi] = a; }
+        }
+        __syncthreads();
       }
+    }
+
+    // how many to keep
+    long long n;
+    if (topk != nullptr) {
+      const float t = topk[h] * (float)nk;     // binary32 product, truncated (utils.py:405)
+      n = (long long)t;
+    } else {
+      // cdf[i] = T(sum_{u<=i} p_sorted[u]);  n = #{i < nk : cdf[i] <= threshold}  (utils.py:398-403)
+      const int seg = nkp / 256;
+      const int p0 = tid * seg;
+      double lsum = 0.0;
+      for (int u = 0; u < seg; u++) lsum += (double)elem_to_f32<DT>((uint16_t)(skey[p0 + u] >> 16));
+      s_tsum[tid] = lsum;
       __syncthreads();
+      double run = 0.0;
+      for (int u = 0; u < tid; u++) run += s_tsum[u];
+      const double thr = (double)cdfthr[h];
+      int cnt = 0;
+      for (int u = 0; u < seg; u++) {
+        run += (double)elem_to_f32<DT>((uint16_t)(skey[p0 + u] >> 16));
+        const float cdfv = elem_to_f32<DT>(f64_to_elem<DT>(run));
+        if (p0 + u < nk && (double)cdfv <= thr) cnt++;
+      }
+      cnt = wave_sum_i32(cnt);
+      if (tid == 0) s_n = 0;
+      __syncthreads();
+      if ((tid & 63) == 0) atomicAdd(&s_n, cnt);
+      __syncthreads();
+      n = s_n;
     }
-  }
+    if (n <= 0) n = 1;                              // utils.py:289
+    const uint32_t kth = (n >= nk) ? 0u : skey[n - 1];
+    __syncthreads();                                // skey is dead from here
 
-  // ---- how many to keep -------------------------------------------------------------------------------
-  long long n;
-  if (topk != nullptr) {
-    const float t = topk[h] * (float)nk;     // binary32 product, truncated (utils.py:405)
-    n = (long long)t;
-  } else {
-    // cdf[i] = T(sum_{u<=i} p_sorted[u]);  n = #{i < nk : cdf[i] <= threshold}  (utils.py:398-403)
-    const int seg = nkp / 256;
-    const int i0 = tid * seg;
-    double lsum = 0.0;
-    for (int u = 0; u < seg; u++) lsum += (double)elem_to_f32<DT>((uint16_t)(skey[i0 + u] >> 16));
-    s_tsum[tid] = lsum;
-    __syncthreads();
-    double run = 0.0;
-    for (int u = 0; u < tid; u++) run += s_tsum[u];
-    const double thr = (double)cdfthr[h];
-    int cnt = 0;
-    for (int u = 0; u < seg; u++) {
-      run += (double)elem_to_f32<DT>((uint16_t)(skey[i0 + u] >> 16));
-      const float cdfv = elem_to_f32<DT>(f64_to_elem<DT>(run));
-      if (i0 + u < nk && (double)cdfv <= thr) cnt++;
-    }
-    cnt = wave_sum_i32(cnt);
-    if (tid == 0) s_n = 0;
-    __syncthreads();
-    if ((tid & 63) == 0) atomicAdd(&s_n, cnt);
-    __syncthreads();
-    n = s_n;
+    // block map row and LUT
+    const bool row_forced = sim_q[(size_t)bh * nq + i] == 0;
+    auto flag = [&](int j) -> bool {
+      bool f = row_forced || (okey[j] >= kth) || (simk[j] == 0);
+      if (j >= causal_lim) f = false;
+      if (sink && j == 0) f = true;
+      return f;
+    };
+    const size_t row_off = ((size_t)bh * nq + i) * nk;
+    if (bmap != nullptr)
+      for (int j = tid; j < nk; j += 256) bmap[row_off + j] = flag(j) ? 1 : 0;
+    emit_lut(flag, nk, nkp, s_idx, s_tmp, lut + row_off, valid + (size_t)bh * nq + i);
+    __syncthreads();                                // the work area is reused by the next row
   }
-  if (n <= 0) n = 1;                              // utils.py:289
-  const uint32_t kth = (n >= nk) ? 0u : skey[n - 1];
-  __syncthreads();                                // skey is dead from here; s_idx may overwrite e_buf's upper half
-
-  // ---- block map row and LUT ---------------------------------------------------------------------------
-  const bool row_forced = sim_q[(size_t)bh * nq + i] == 0;
-  auto flag = [&](int j) -> bool {
-    bool f = row_forced || (okey[j] >= kth) || (simk[j] == 0);
-    if (j >= causal_lim) f = false;
-    if (sink && j == 0) f = true;
-    return f;
-  };
-  const size_t row_off = ((size_t)bh * nq + i) * nk;
-  if (bmap != nullptr)
-    for (int j = tid; j < nk; j += 256) bmap[row_off + j] = flag(j) ? 1 : 0;
-  emit_lut(flag, nk, nkp, s_idx, s_tmp, lut + row_off, valid + (size_t)bh * nq + i);
 }
 
 // =============================================================================================
@@ -541,20 +560,30 @@ void launch_pool_sim_quant(const void *x, const void *km, void *pool, uint8_t *s
 
 int block_select_max_nk() { return 8192; }
 
+template <int D, int DT, int R>
+static hipError_t launch_bs3(const void *pq, const uint8_t *sq, const void *pk, const uint8_t *sk, const float *topk,
+                             const float *cdf, int causal, int sink, int32_t *lut, int32_t *valid, uint8_t *bmap, int B,
+                             int H, int nq, int nk, int nkp, hipStream_t st) {
+  const size_t lds = (size_t)R * D * 8 + (size_t)R * nkp * 4 + 12 * (size_t)nkp;
+  auto kern = block_select_kernel<D, DT, R>;
+  if (lds > 48 * 1024) {
+    hipError_t e = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    if (e != hipSuccess) return e;
+  }
+  kern<<<dim3((nq + R - 1) / R, B * H), 256, lds, st>>>((const uint16_t *)pq, sq, (const uint16_t *)pk, sk, topk, cdf,
+                                                        causal, sink, lut, valid, bmap, H, nq, nk, nkp);
+  return hipSuccess;
+}
+
 template <int D, int DT>
 static hipError_t launch_bs2(const void *pq, const uint8_t *sq, const void *pk, const uint8_t *sk, const float *topk,
                              const float *cdf, int causal, int sink, int32_t *lut, int32_t *valid, uint8_t *bmap, int B,
                              int H, int nq, int nk, hipStream_t st) {
   const int nkp = next_pow2_ge(nk, 256);
-  const size_t lds = 12 * (size_t)nkp;
-  auto kern = block_select_kernel<D, DT>;
-  if (lds > 48 * 1024) {
-    hipError_t e = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-    if (e != hipSuccess) return e;
-  }
-  kern<<<dim3(nq, B * H), 256, lds, st>>>((const uint16_t *)pq, sq, (const uint16_t *)pk, sk, topk, cdf, causal, sink, lut,
-                                         valid, bmap, H, nq, nk, nkp);
-  return hipSuccess;
+  // rows per workgroup: reuse of the pooled-K reads against LDS footprint (scores are R*nkp floats)
+  if (nkp <= 1024) return launch_bs3<D, DT, 8>(pq, sq, pk, sk, topk, cdf, causal, sink, lut, valid, bmap, B, H, nq, nk, nkp, st);
+  if (nkp <= 4096) return launch_bs3<D, DT, 4>(pq, sq, pk, sk, topk, cdf, causal, sink, lut, valid, bmap, B, H, nq, nk, nkp, st);
+  return launch_bs3<D, DT, 2>(pq, sq, pk, sk, topk, cdf, causal, sink, lut, valid, bmap, B, H, nq, nk, nkp, st);
 }
 
 hipError_t launch_block_select(const void *pq, const uint8_t *sq, const void *pk, const uint8_t *sk, const float *topk,
