@@ -23,6 +23,10 @@ sys.path.insert(0, ROOT)
 
 PEAK_MFMA_8BIT = 5.0e15   # MI355X dense INT8 = FP8 MFMA peak, op/s
 PEAK_HBM = 8.0e12
+# HBM-side bytes per launch of the attention kernel, measured with two rocprofv3 --pmc runs (FETCH_SIZE, WRITE_SIZE,
+# each scaled by what the same counter reads for a 1 GiB device copy: x2.0 and x1.0).  Only known for the workload
+# it was measured on.
+MEASURED_ATTN_TRAFFIC = {"cfg4": int((1.72 + 0.25) * 2 ** 30)}
 
 
 def parse():
@@ -33,6 +37,9 @@ def parse():
     ap.add_argument("--config", default="cfg4", help="workload (cfg1..cfg5); the headline is cfg4")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-dense", action="store_true")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="run only a 1 GiB device-to-device copy (known traffic) - the reference point for scaling the "
+                         "FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run")
     ap.add_argument("--attn-only", action="store_true",
                     help="time only the attention kernel launches (for rocprofv3 runs of the dominant kernel)")
     return ap.parse_args()
@@ -64,6 +71,17 @@ def main():
         sys.exit(2)
     import spargeattn_amd as sa
     from spargeattn_amd import core, _lib, workloads as W
+
+    if args.copy_calibration:
+        torch.cuda.set_device(0)
+        n = 1 << 30
+        a = torch.empty(n, dtype=torch.uint8, device="cuda")
+        b = torch.zeros(n, dtype=torch.uint8, device="cuda")
+        for _ in range(3):
+            a.copy_(b)
+        torch.cuda.synchronize()
+        print(json.dumps({"copy_bytes_read": n, "copy_bytes_written": n}))
+        return
 
     cfg = W.CONFIGS[args.config]
     if cfg.api != "topk":
@@ -170,7 +188,7 @@ def main():
         "v_quant": {"us": stage_ms["vquant"] * 1e3, "GBps": vq_bytes / (stage_ms["vquant"] * 1e-3) / 1e9},
         "roofline": {"kernel": "block_sparse_attn_kernel<128,bf16>", "bound": "mfma",
                      "achieved": executed_ops / attn_s / 1e12, "peak": PEAK_MFMA_8BIT / 1e12, "unit": "TFLOP/s",
-                     "frac": executed_ops / attn_s / PEAK_MFMA_8BIT, "traffic": None,
+                     "frac": executed_ops / attn_s / PEAK_MFMA_8BIT, "traffic": MEASURED_ATTN_TRAFFIC.get(cfg.name),
                      "note": "achieved = executed INT8+FP8 MFMA ops (selected blocks * 2*128*64*D*2) / HIP-event time of "
                              "the kernel inside the timed steps; peak = MI355X dense 8-bit MFMA"},
     }
