@@ -50,25 +50,28 @@ __global__ __launch_bounds__(256, 2) void dense_attn_f16_kernel(const DenseParam
   const uint16_t *vbase = p.vt + (size_t)bh * p.nk * (size_t)(D * 64);
   const float c = p.sm_scale_log2;
 
-  uint4 kr[CH], vr[CH];
-  auto fetch = [&](int blk) {
-#pragma unroll
-    for (int u = 0; u < CH; u++) {
-      const int ci = tid + 256 * u;
-      const int row = ci / (D / 8), col = ci % (D / 8);
-      kr[u] = make_uint4(0, 0, 0, 0);
-      if (blk * 64 + row < N) kr[u] = *(const uint4 *)(kbase + ((size_t)blk * 64 + row) * D + col * 8);
-      vr[u] = *(const uint4 *)(vbase + (size_t)blk * (D * 64) + (size_t)ci * 8);
-    }
-  };
-  auto stash = [&](int buf) {
-#pragma unroll
-    for (int u = 0; u < CH; u++) {
-      const int ci = tid + 256 * u;
-      *(uint4 *)(sKp(buf) + (ci / (D / 8)) * KSTR + (ci % (D / 8)) * 16) = kr[u];
-      *(uint4 *)(sVp(buf) + (ci >> 3) * VSTR + (ci & 7) * 16) = vr[u];
-    }
-  };
+  // staging registers for the next block's tiles (named scalars: an indexed array ends up in scratch memory)
+  uint4 kr0, kr1, kr2, kr3, vr0, vr1, vr2, vr3;
+  kr0 = kr1 = kr2 = kr3 = vr0 = vr1 = vr2 = vr3 = make_uint4(0, 0, 0, 0);
+#define SPG_FETCH1(U, KR, VR, BLK)                                                                       \
+  if constexpr (CH > U) {                                                                                \
+    const int ci = tid + 256 * U;                                                                        \
+    const int row = ci / (D / 8), col = ci % (D / 8);                                                    \
+    /* rows beyond N (last block only) are clamped to a valid row: their scores are masked below */      \
+    const int grow = min((BLK) * 64 + row, N - 1);                                                       \
+    KR = *(const uint4 *)(kbase + (size_t)grow * D + col * 8);                                           \
+    VR = *(const uint4 *)(vbase + (size_t)(BLK) * (D * 64) + (size_t)ci * 8);                            \
+  }
+#define SPG_FETCH(BLK)                                                                                   \
+  { SPG_FETCH1(0, kr0, vr0, BLK) SPG_FETCH1(1, kr1, vr1, BLK) SPG_FETCH1(2, kr2, vr2, BLK) SPG_FETCH1(3, kr3, vr3, BLK) }
+#define SPG_STASH1(U, KR, VR, BUF)                                                                       \
+  if constexpr (CH > U) {                                                                                \
+    const int ci = tid + 256 * U;                                                                        \
+    *(uint4 *)(sKp(BUF) + (ci / (D / 8)) * KSTR + (ci % (D / 8)) * 16) = KR;                             \
+    *(uint4 *)(sVp(BUF) + (ci >> 3) * VSTR + (ci & 7) * 16) = VR;                                        \
+  }
+#define SPG_STASH(BUF)                                                                                   \
+  { SPG_STASH1(0, kr0, vr0, BUF) SPG_STASH1(1, kr1, vr1, BUF) SPG_STASH1(2, kr2, vr2, BUF) SPG_STASH1(3, kr3, vr3, BUF) }
 
   // MFMA row i of key tile kt carries key 32*kt + 16*(i>>4) + 8*((i>>2)&1) + 4*((i>>3)&1) + (i&3):
   // after S^T, the 8 registers [8n', 8n'+8) of a lane hold 8 consecutive keys 16*(2kt+n') + 8*half + (0..7).
@@ -81,8 +84,8 @@ __global__ __launch_bounds__(256, 2) void dense_attn_f16_kernel(const DenseParam
 #pragma unroll
     for (int e = 0; e < 16; e++) O[dt][e] = 0.f;
 
-  fetch(0);
-  stash(0);
+  SPG_FETCH(0);
+  SPG_STASH(0);
   int buf = 0;
   for (int blk = 0; blk < nblk; blk++) {
     __syncthreads();
@@ -98,7 +101,7 @@ __global__ __launch_bounds__(256, 2) void dense_attn_f16_kernel(const DenseParam
       }
     }
     const bool more = blk + 1 < nblk;
-    if (more) fetch(blk + 1);
+    SPG_FETCH(more ? blk + 1 : blk);   // unconditional: keeps the staging registers out of scratch
 
     // register e of tile kt <-> key 64*blk + 32*kt + 16*(e>>3) + 8*hh + (e&7)
     const bool edge = (p.is_causal && blk >= 2 * qb) || (blk == p.nk - 1);
@@ -115,7 +118,7 @@ __global__ __launch_bounds__(256, 2) void dense_attn_f16_kernel(const DenseParam
         }
         fm = fmaxf(fm, v);
       }
-    fm = fmaxf(fm, __shfl_xor(fm, 32, SPG_WAVE)) * c;
+    fm = half_swap_max_f32(fm) * c;
     const float m_new = fmaxf(m, fm);
     const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
     const float osc = __builtin_amdgcn_exp2f(m - m_use);
@@ -132,10 +135,13 @@ __global__ __launch_bounds__(256, 2) void dense_attn_f16_kernel(const DenseParam
 #pragma unroll
     for (int kt = 0; kt < 2; kt++)
 #pragma unroll
-      for (int e = 0; e < 16; e++) {
-        const float pv = __builtin_amdgcn_exp2f(__builtin_fmaf(S[kt][e], c, -m_use));
-        ps += pv;
-        pb[2 * kt + (e >> 3)][e & 7] = (_Float16)pv;
+      for (int e = 0; e < 16; e += 2) {
+        const float p0 = __builtin_amdgcn_exp2f(__builtin_fmaf(S[kt][e], c, -m_use));
+        const float p1 = __builtin_amdgcn_exp2f(__builtin_fmaf(S[kt][e + 1], c, -m_use));
+        ps += p0 + p1;
+        const auto h2 = __builtin_amdgcn_cvt_pkrtz(p0, p1);      // two fp16 in one instruction
+        pb[2 * kt + (e >> 3)][e & 7] = (_Float16)h2[0];
+        pb[2 * kt + (e >> 3)][(e & 7) + 1] = (_Float16)h2[1];
       }
     dsum += ps;
 #pragma unroll
@@ -146,11 +152,15 @@ __global__ __launch_bounds__(256, 2) void dense_attn_f16_kernel(const DenseParam
         O[dt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(v8h, t), pb[n], O[dt], 0, 0, 0);
       }
     }
-    if (more) stash(buf ^ 1);   // buf^1 was last read before this iteration's barrier
+    SPG_STASH(buf ^ 1);                // buf^1 was last read before this iteration's barrier
     buf ^= 1;
   }
 
-  const float dtot = dsum + __shfl_xor(dsum, 32, SPG_WAVE);
+#undef SPG_FETCH
+#undef SPG_STASH
+#undef SPG_FETCH1
+#undef SPG_STASH1
+  const float dtot = half_swap_sum_f32(dsum);
   const float inv = 1.0f / dtot;
   if (q_row < N) {
     uint16_t *orow = p.out + ((size_t)bh * N + q_row) * D;
