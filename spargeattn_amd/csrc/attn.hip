@@ -50,6 +50,23 @@ struct AttnParams {
   int total_wg, wg_per_xcd;
 };
 
+// LDS tile reads are issued through inline asm with explicit waits.  Left to the compiler, every LDS read would be
+// ordered after ALL outstanding direct-to-LDS loads of the ring (s_waitcnt vmcnt(0)), which serialises the prefetch
+// of block it+2 with the compute of block it.  The ring's own protocol (vmcnt(0) + barrier before a slot is read)
+// is what guarantees correctness.
+template <int OFF0, int OFF1>
+__device__ __forceinline__ void lds_read_2x128(v4i &a, v4i &b, uint32_t addr) {
+  asm volatile("ds_read_b128 %0, %2 offset:%3\n\tds_read_b128 %1, %2 offset:%4"
+               : "=&v"(a), "=&v"(b)
+               : "v"(addr), "n"(OFF0), "n"(OFF1)
+               : "memory");
+}
+// wait for all outstanding LDS reads; the operands tie the wait to the registers it makes valid
+__device__ __forceinline__ void lds_wait4(v4i &a, v4i &b, v4i &c, v4i &d) {
+  asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(a), "+v"(b), "+v"(c), "+v"(d));
+}
+__device__ __forceinline__ void lds_wait2(v4i &a, v4i &b) { asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(a), "+v"(b)); }
+
 // 16-byte-chunk swizzles.  K tile row = key (D bytes, D/16 chunks); V^T tile row = channel (64 bytes, 4 chunks).
 // The functions are chosen such that any 8 consecutive lanes of a ds_read_b128 hit 8 different 16-byte bank groups.
 template <int D>
@@ -72,6 +89,8 @@ __global__ __launch_bounds__(256, 3) void block_sparse_attn_kernel(const AttnPar
   __shared__ int sVote[2][4];
   unsigned char *const sKr = smem;
   unsigned char *const sVr = smem + NBUF * TILE;
+  const uint32_t lds_k0 = (uint32_t)(size_t)(__attribute__((address_space(3))) unsigned char *)smem;   // LDS byte address
+  const uint32_t lds_v0 = lds_k0 + NBUF * TILE;
 
   // ---- workgroup -> (batch*head, q block): one XCD per head at a time, heavy (late) rows first ----------
   const int w = blockIdx.x;
@@ -182,12 +201,10 @@ __global__ __launch_bounds__(256, 3) void block_sparse_attn_kernel(const AttnPar
   if (nv > 1) SPG_LOAD_TILES(blk1, TILE);
   uint32_t bufoff = 0;                     // LDS ring offset of block it
 
+  __builtin_amdgcn_s_waitcnt(0x0F70);     // vmcnt(0): Q fragment and the first tiles have arrived
+  __syncthreads();
 #pragma unroll 1
   for (int it = 0; it < nv; it++) {
-    if (it == 0) {
-      __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0)
-      __syncthreads();
-    }
     // scalar prefetches for later iterations (SMEM)
     const float ksc2 = kscale[blk2];
     const int d4 = it + 4 < nv ? lutc[it + 4] : 0;
@@ -196,14 +213,27 @@ __global__ __launch_bounds__(256, 3) void block_sparse_attn_kernel(const AttnPar
     v16i S0, S1;
 #pragma unroll
     for (int e = 0; e < 16; e++) { S0[e] = 0; S1[e] = 0; }
-    const unsigned char *kt = sKr + bufoff;
+    {
+      // two groups of k-steps: the reads of the second group are in flight while the first group's MFMAs run
+      constexpr int HK = KS / 2;
+      const uint32_t kaddr = lds_k0 + bufoff + k_rd_base;
+      v4i a0[KS], a1[KS];
 #pragma unroll
-    for (int ks = 0; ks < KS; ks++) {
-      const uint32_t ko = k_rd_base + ((uint32_t)(32 * ks) ^ k_rd_x);
-      const v4i a0 = *(const v4i *)(kt + ko);
-      const v4i a1 = *(const v4i *)(kt + ko + 16 * D);
-      S0 = __builtin_amdgcn_mfma_i32_32x32x32_i8(a0, qreg[ks], S0, 0, 0, 0);
-      S1 = __builtin_amdgcn_mfma_i32_32x32x32_i8(a1, qreg[ks], S1, 0, 0, 0);
+      for (int ks = 0; ks < HK; ks++) lds_read_2x128<0, 16 * D>(a0[ks], a1[ks], kaddr + ((uint32_t)(32 * ks) ^ k_rd_x));
+      if constexpr (HK == 2) lds_wait4(a0[0], a1[0], a0[1], a1[1]); else lds_wait2(a0[0], a1[0]);
+#pragma unroll
+      for (int ks = HK; ks < KS; ks++) lds_read_2x128<0, 16 * D>(a0[ks], a1[ks], kaddr + ((uint32_t)(32 * ks) ^ k_rd_x));
+#pragma unroll
+      for (int ks = 0; ks < HK; ks++) {
+        S0 = __builtin_amdgcn_mfma_i32_32x32x32_i8(a0[ks], qreg[ks], S0, 0, 0, 0);
+        S1 = __builtin_amdgcn_mfma_i32_32x32x32_i8(a1[ks], qreg[ks], S1, 0, 0, 0);
+      }
+      if constexpr (HK == 2) lds_wait4(a0[2], a1[2], a0[3], a1[3]); else lds_wait2(a0[1], a1[1]);
+#pragma unroll
+      for (int ks = HK; ks < KS; ks++) {
+        S0 = __builtin_amdgcn_mfma_i32_32x32x32_i8(a0[ks], qreg[ks], S0, 0, 0, 0);
+        S1 = __builtin_amdgcn_mfma_i32_32x32x32_i8(a1[ks], qreg[ks], S1, 0, 0, 0);
+      }
     }
 
     const float dq = qs * ksc;
@@ -249,13 +279,13 @@ __global__ __launch_bounds__(256, 3) void block_sparse_attn_kernel(const AttnPar
     }
     __builtin_amdgcn_s_waitcnt(0x0F70);   // this wave's share of block it+1's tiles has landed in LDS
     __syncthreads();   // block it+1's tiles are complete; the votes are visible; ring slot of block it-1 is free
+    bool compute = true;
+    if (!tail)         // workgroup-uniform (PVThresholdMode::kPerBlock, sm89.cuh:318-353)
+      compute = (sVote[it & 1][0] | sVote[it & 1][1] | sVote[it & 1][2] | sVote[it & 1][3]) != 0;
     if (it + 2 < nv) {
       const uint32_t b2 = bufoff == 0 ? 2 * TILE : bufoff - TILE;   // slot (it+2) % 3
       SPG_LOAD_TILES(blk2, b2);
     }
-    bool compute = true;
-    if (!tail)         // workgroup-uniform (PVThresholdMode::kPerBlock, sm89.cuh:318-353)
-      compute = (sVote[it & 1][0] | sVote[it & 1][1] | sVote[it & 1][2] | sVote[it & 1][3]) != 0;
     dsum *= osc;
     if (__any(osc != 1.0f)) {
 #pragma unroll
@@ -276,19 +306,41 @@ __global__ __launch_bounds__(256, 3) void block_sparse_attn_kernel(const AttnPar
       v8i pb;
 #pragma unroll
       for (int u = 0; u < 8; u++) {
-        // both halves of the destination are written: the initial content is irrelevant, so the register of
-        // x[4u] is reused instead of a zeroed one
-        int wv = __builtin_amdgcn_cvt_pk_fp8_f32(x[4 * u], x[4 * u + 1], __builtin_bit_cast(int, x[4 * u]), false);
+        // both halves of the destination are written, so its initial content is irrelevant: start from a register
+        // that is "defined" by an empty asm instead of a zeroed one
+        int wv;
+        asm volatile("" : "=v"(wv));
+        wv = __builtin_amdgcn_cvt_pk_fp8_f32(x[4 * u], x[4 * u + 1], wv, false);
         wv = __builtin_amdgcn_cvt_pk_fp8_f32(x[4 * u + 2], x[4 * u + 3], wv, true);
         pb[u] = wv;
       }
-      const unsigned char *vt = sVr + bufoff;
+      {
+        constexpr int HD = NDT / 2;
+        const uint32_t va_lo = lds_v0 + bufoff + v_rd_lo, va_hi = lds_v0 + bufoff + (v_rd_lo ^ 16u);
+        v4i lo[NDT], hi[NDT];
+        // group 0
+        asm volatile("ds_read_b128 %0, %2\n\tds_read_b128 %1, %3" : "=&v"(lo[0]), "=&v"(hi[0]) : "v"(va_lo), "v"(va_hi) : "memory");
+        if constexpr (HD == 2)
+          asm volatile("ds_read_b128 %0, %2 offset:2048\n\tds_read_b128 %1, %3 offset:2048" : "=&v"(lo[1]), "=&v"(hi[1]) : "v"(va_lo), "v"(va_hi) : "memory");
+        if constexpr (HD == 2) lds_wait4(lo[0], hi[0], lo[1], hi[1]); else lds_wait2(lo[0], hi[0]);
+        // group 1 in flight while group 0 multiplies
+        if constexpr (HD == 2) {
+          asm volatile("ds_read_b128 %0, %2 offset:4096\n\tds_read_b128 %1, %3 offset:4096" : "=&v"(lo[2]), "=&v"(hi[2]) : "v"(va_lo), "v"(va_hi) : "memory");
+          asm volatile("ds_read_b128 %0, %2 offset:6144\n\tds_read_b128 %1, %3 offset:6144" : "=&v"(lo[3]), "=&v"(hi[3]) : "v"(va_lo), "v"(va_hi) : "memory");
+        } else {
+          asm volatile("ds_read_b128 %0, %2 offset:2048\n\tds_read_b128 %1, %3 offset:2048" : "=&v"(lo[1]), "=&v"(hi[1]) : "v"(va_lo), "v"(va_hi) : "memory");
+        }
 #pragma unroll
-      for (int dt = 0; dt < NDT; dt++) {
-        const v4i lo = *(const v4i *)(vt + v_rd_lo + dt * 2048);
-        const v4i hi = *(const v4i *)(vt + (v_rd_lo ^ 16u) + dt * 2048);
-        const v8i av = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-        O[dt] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(av, pb, O[dt], 0, 0, 0, 0, 0, 0);
+        for (int dt = 0; dt < HD; dt++) {
+          const v8i av = {lo[dt][0], lo[dt][1], lo[dt][2], lo[dt][3], hi[dt][0], hi[dt][1], hi[dt][2], hi[dt][3]};
+          O[dt] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(av, pb, O[dt], 0, 0, 0, 0, 0, 0);
+        }
+        if constexpr (HD == 2) lds_wait4(lo[2], hi[2], lo[3], hi[3]); else lds_wait2(lo[1], hi[1]);
+#pragma unroll
+        for (int dt = HD; dt < NDT; dt++) {
+          const v8i av = {lo[dt][0], lo[dt][1], lo[dt][2], lo[dt][3], hi[dt][0], hi[dt][1], hi[dt][2], hi[dt][3]};
+          O[dt] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(av, pb, O[dt], 0, 0, 0, 0, 0, 0);
+        }
       }
     }
     // advance the block pipeline and the ring
