@@ -1,0 +1,156 @@
+"""Full-size GPU checks on the BASELINE configurations through size-independent properties.
+
+The oracle is too slow at these sizes; instead each test checks invariants the algorithm fixes (row counts of the
+block map, LUT sortedness, quantisation round-trip bounds, code-range of the FP8 tensor, determinism) and compares
+sampled Q blocks of the attention output with a float32 torch computation on the de-quantised tensors under the
+token mask the LUT encodes.
+"""
+import numpy as np
+import pytest
+import torch
+
+import spargeattn_amd as sa
+from spargeattn_amd import _lib, utils, workloads as W
+
+pytestmark = pytest.mark.gpu
+
+
+def _lut_to_map(lut, valid):
+    """delta LUT -> boolean block map (on the GPU)."""
+    B, H, nq, nk = lut.shape
+    idx = torch.cumsum(lut.long(), dim=-1)
+    sel = torch.arange(nk, device=lut.device)[None, None, None, :] < valid[..., None]
+    m = torch.zeros((B, H, nq, nk + 1), dtype=torch.bool, device=lut.device)
+    m.scatter_(3, torch.where(sel, idx, torch.full_like(idx, nk)), True)
+    return m[..., :nk], idx, sel
+
+
+def _reference_rows(q8, qs, k8, ks, v8_nat, vs, bmap, b, h, qb, N, D, causal_tokens=False):
+    """float32 attention of one Q block on the de-quantised tensors under the block mask."""
+    r0, r1 = qb * 128, min(N, qb * 128 + 128)
+    q = q8[b, h, r0:r1].float() * qs[b, h, qb]
+    k = k8[b, h].float() * ks[b, h].repeat_interleave(64)[:N, None]
+    v = _lib_e4m3_to_float(v8_nat[b, h, :N]) * vs[b, h][None, :]
+    s = (q @ k.T) * (D ** -0.5)
+    tm = bmap[b, h, qb].repeat_interleave(64)[:N]
+    s = s.masked_fill(~tm[None, :], float("-inf"))
+    if causal_tokens:
+        rows = torch.arange(r0, r1, device=s.device)[:, None]
+        s = s.masked_fill(torch.arange(N, device=s.device)[None, :] > rows, float("-inf"))
+    return torch.softmax(s, dim=-1) @ v
+
+
+def _lib_e4m3_to_float(codes):
+    return codes.view(torch.float8_e4m3fn).float()
+
+
+def _cos_l1(a, b):
+    a, b = a.double().flatten(), b.double().flatten()
+    return (torch.dot(a, b) / (a.norm() * b.norm())).item(), ((a - b).abs().sum() / b.abs().sum()).item()
+
+
+def _check_quant(x, xq, scale, bs):
+    """|x - q*s| <= s/2 (+ rounding slack) and every block reaches |q| = 127 unless the 1e-7 term matters."""
+    B, H, N, D = x.shape
+    s_tok = scale.repeat_interleave(bs, dim=2)[:, :, :N, None]
+    err = (x.float() - xq.float() * s_tok).abs()
+    assert bool((err <= 0.5 * s_tok * (1 + 1e-4)).all())
+    nb = scale.shape[2]
+    pad = nb * bs - N
+    q = torch.nn.functional.pad(xq, (0, 0, 0, pad)).view(B, H, nb, bs * D).abs().amax(dim=-1)
+    assert int(q.max()) == 127 and int(q.min()) >= 126
+
+
+@pytest.mark.parametrize("name", ["cfg4", "cfg3", "cfg5"])
+def test_topk_operator_full_size(name):
+    cfg = W.CONFIGS[name]
+    torch.manual_seed(0)
+    q, k, v = W.make_qkv(cfg, device="cuda")
+    B, H, N, D = q.shape
+    nq, nk = (N + 127) // 128, (N + 63) // 64
+
+    km = _lib.km_mean(k)
+    ref_km = k.double().mean(dim=-2, keepdim=True)
+    assert float((km.double() - ref_km).abs().max()) <= float(ref_km.abs().max()) * 2.0 ** -8 + 1e-6
+
+    lut, valid, q8, qs, k8, ks = utils.get_block_map_meansim_fuse_quant(
+        q, k, km, is_causal=cfg.is_causal, simthreshd1=-0.1, cdfthreshd=None, topk=cfg.topk, return_lut=True)
+    bmap2, *_ = utils.get_block_map_meansim_fuse_quant(
+        q, k, km, is_causal=cfg.is_causal, simthreshd1=-0.1, cdfthreshd=None, topk=cfg.topk, return_lut=False)
+    bmap, idx, sel = _lut_to_map(lut, valid)
+    assert torch.equal(bmap, bmap2)                                   # LUT and map outputs describe the same set
+    # ascending, in range, zero tail
+    assert bool(((lut > 0) | ~sel | (torch.arange(nk, device="cuda") == 0)).all())
+    assert bool((idx[sel] < nk).all()) and bool((lut[~sel] == 0).all())
+    assert torch.equal(valid.long(), bmap.sum(-1))
+    # row counts fixed by the algorithm (all full blocks are "similar" at simthreshd1 = -0.1)
+    n_sel = max(1, int(np.float32(cfg.topk) * np.float32(nk)))
+    counts = valid.long()
+    full_rows = nq if N % 128 == 0 else nq - 1
+    if cfg.is_causal:
+        want = torch.minimum(2 * (torch.arange(nq, device="cuda") + 1), torch.tensor(n_sel, device="cuda"))
+        assert bool((counts == want[None, None, :]).all())
+        assert not bool((bmap & ~(torch.arange(nk, device="cuda")[None, :] < 2 * (torch.arange(nq, device="cuda")[:, None] + 1))).any())
+    else:
+        forced = 0 if N % 64 == 0 else 1                               # the partial last K block is never skipped
+        c = counts[:, :, :full_rows]
+        assert bool(((c == n_sel) | (c == n_sel + forced)).all())
+        if forced:
+            assert bool(bmap[..., nk - 1].all())
+        if full_rows < nq:
+            assert bool((counts[:, :, -1] == nk).all())                # partial last Q block keeps every column
+    expect_sparsity = 1 - float(valid.float().sum()) / ((((nk + 2) // 2) if cfg.is_causal else nk) * nq * B * H)
+
+    _check_quant(q, q8, qs, 128)
+    ksm = (k.float() - km.float()).to(k.dtype)                         # (k - km) in the input dtype
+    _check_quant(ksm, k8, ks, 64)
+
+    v8, vs = _lib.v_quant_fp8(v)
+    nat = _lib.v8_tiles_to_natural(v8)
+    assert bool((nat[:, :, N:] == 0).all())
+    dec = _lib_e4m3_to_float(nat[:, :, :N])
+    assert float(dec.abs().amax(dim=2).min()) == 2.25 and float(dec.abs().max()) == 2.25
+    v16 = v.to(torch.float16).float()
+    assert torch.allclose(vs, v16.abs().amax(dim=2) / 2.25, rtol=3e-7, atol=0)
+
+    o, sparsity = sa.spas_sage2_attn_meansim_topk_cuda(q, k, v, is_causal=cfg.is_causal, topk=cfg.topk,
+                                                       pvthreshd=cfg.pvthreshd, return_sparsity=True)
+    assert abs(sparsity - expect_sparsity) < 1e-5
+    assert o.shape == q.shape and o.dtype == cfg.dtype and bool(torch.isfinite(o.float()).all())
+    o2 = sa.spas_sage2_attn_meansim_topk_cuda(q, k, v, is_causal=cfg.is_causal, topk=cfg.topk, pvthreshd=cfg.pvthreshd)
+    assert torch.equal(o, o2)                                          # deterministic
+    # sampled Q blocks against float32 attention on the de-quantised tensors under the same block mask
+    for (h, qb) in [(0, 0), (H // 2, nq // 3), (H - 1, nq - 1), (1, nq // 2)]:
+        ref = _reference_rows(q8, qs, k8, ks, nat, vs, bmap, 0, h, qb, N, D)
+        cos, l1 = _cos_l1(o[0, h, qb * 128:qb * 128 + ref.shape[0]].float(), ref)
+        print(f"{name} head {h} q-block {qb}: cos {cos:.6f} rel-L1 {l1:.4f}", flush=True)
+        assert cos >= 0.999 and l1 <= 3e-2, (name, h, qb, cos, l1)     # residual: e4m3 rounding of P, bf16 output
+    # executed PV count equals the number of selected blocks at threshold 50
+    pvt = torch.full((H,), float(cfg.pvthreshd), device="cuda")
+    o3 = torch.empty_like(q)
+    pvc = _lib.block_sparse_attn(q8, k8, v8, o3, lut, valid, pvt, qs, ks, vs, D ** -0.5, return_pv_count=True)
+    assert torch.equal(pvc, valid) and torch.equal(o3, o)
+
+
+def test_mask_operator_full_size_cfg2():
+    cfg = W.CONFIGS["cfg2"]
+    q, k, v = W.make_qkv(cfg, device="cuda")
+    B, H, N, D = q.shape
+    nq, nk = (N + 127) // 128, (N + 63) // 64
+    mask = W.make_mask_id(cfg, B, H, N, device="cuda")
+    assert mask.shape == (B, H, nq, nk)
+    lut, valid = utils.block_map_lut_triton(mask)
+    bmap, idx, sel = _lut_to_map(lut, valid)
+    assert torch.equal(bmap, mask.bool()) and torch.equal(valid.long(), mask.bool().sum(-1))
+    o, sparsity = sa.block_sparse_sage2_attn_cuda(q, k, v, mask_id=mask, return_sparsity=True)
+    assert abs(sparsity - (1 - float(valid.float().sum()) / (((nk + 2) // 2) * nq * B * H))) < 1e-5
+    assert bool(torch.isfinite(o.float()).all())
+    # masked fp32 reference on the ORIGINAL tensors for sampled Q blocks (what this configuration is specified against)
+    for (b, h, qb) in [(0, 0, 0), (1, H - 1, nq - 1), (0, 7, nq // 2)]:
+        r0 = qb * 128
+        s = (q[b, h, r0:r0 + 128].float() @ k[b, h].float().T) * D ** -0.5
+        tm = mask[b, h, qb].bool().repeat_interleave(64)[:N]
+        ref = torch.softmax(s.masked_fill(~tm[None, :], float("-inf")), dim=-1) @ v[b, h].float()
+        cos, l1 = _cos_l1(o[b, h, r0:r0 + 128].float(), ref)
+        print(f"cfg2 b{b} h{h} q-block {qb}: cos {cos:.6f} rel-L1 {l1:.4f}", flush=True)
+        assert cos >= 0.995, (b, h, qb, cos, l1)                        # includes the INT8/FP8 quantisation error
