@@ -70,9 +70,9 @@ __device__ __forceinline__ void lds_wait2(v4i &a, v4i &b) { asm volatile("s_wait
 // 16-byte-chunk swizzles.  K tile row = key (D bytes, D/16 chunks); V^T tile row = channel (64 bytes, 4 chunks).
 // The functions are chosen such that any 8 consecutive lanes of a ds_read_b128 hit 8 different 16-byte bank groups.
 template <int D>
-__device__ __forceinline__ int k_swz(int row) {
-  if constexpr (D == 128) return (row & 3) | (((row >> 5) & 1) << 2);
-  else return ((row >> 1) & 1) | (((row >> 5) & 1) << 1);
+__device__ __forceinline__ uint32_t k_swz(uint32_t row) {
+  if constexpr (D == 128) return (row & 3u) | (((row >> 5) & 1u) << 2);
+  else return ((row >> 1) & 1u) | (((row >> 5) & 1u) << 1);
 }
 __device__ __forceinline__ int v_swz(int row) { return (row >> 1) & 3; }
 
@@ -103,7 +103,8 @@ __global__ __launch_bounds__(256, 3) void block_sparse_attn_kernel(const AttnPar
   if (nv == 0) return;                                       // output rows stay unwritten (sm89.cuh:232-235)
   const int32_t *lut_row = p.lut + ((size_t)bh * p.nq + qb) * p.nk;
 
-  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, r = lane & 31, hh = lane >> 5;
+  const int tid = threadIdx.x, lane = tid & 63, r = lane & 31, hh = lane >> 5;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);   // uniform: everything derived from it stays scalar
   const int N = p.N;
   const int q_row = qb * 128 + wave * 32 + r;
 
@@ -134,11 +135,11 @@ __global__ __launch_bounds__(256, 3) void block_sparse_attn_kernel(const AttnPar
   // (the two per-lane offsets are recomputed from the thread id where they are used: cheaper than keeping them
   //  in registers across the loop, where the register file is the scarce resource)
 #define SPG_LANE_OFFSETS()                                                                                    \
-  int tid_ = threadIdx.x;                                                                                     \
-  asm volatile("" : "+v"(tid_));                                                                              \
-  const int pos0 = WL * (tid_ >> 6) * 64 + (tid_ & 63);                                                       \
-  const uint32_t k_lane = (uint32_t)((pos0 / CPR) * D + ((pos0 % CPR) ^ k_swz<D>(pos0 / CPR)) * 16);          \
-  const uint32_t v_lane = (uint32_t)pos0 * 16u;
+  uint32_t lane_ = threadIdx.x & 63u;                                                                         \
+  asm volatile("" : "+v"(lane_));                                                                             \
+  const uint32_t pos0 = (uint32_t)(WL * 64 * wave) + lane_;                                                   \
+  const uint32_t v_lane = pos0 * 16u;                                                                         \
+  const uint32_t k_lane = v_lane ^ (k_swz<D>(pos0 / CPR) * 16u);   /* row * D + (slot ^ swz) * 16 */
   const int last_partial_blk = (N % 64) ? p.nk - 1 : -1;   // the only block with rows beyond N
   typedef __attribute__((address_space(3))) void *lds_ptr_t;
   typedef const __attribute__((address_space(1))) void *glb_ptr_t;
@@ -160,9 +161,9 @@ __global__ __launch_bounds__(256, 3) void block_sparse_attn_kernel(const AttnPar
       /* rows beyond N are clamped to row N-1: their scores are masked, their V rows are zero */              \
       const int rows_ok_ = N - (BLK) * 64;                                                                    \
       _Pragma("unroll") for (int u = 0; u < WL; u++) {                                                        \
-        const int pos = pos0 + u * 64;                                                                        \
-        const int row_ = min(pos / CPR, rows_ok_ - 1);                                                        \
-        const uint32_t ko_ = (uint32_t)(row_ * D + ((pos % CPR) ^ k_swz<D>(pos / CPR)) * 16);                 \
+        const uint32_t pos = pos0 + u * 64;                                                                   \
+        const uint32_t row_ = min(pos / CPR, (uint32_t)(rows_ok_ - 1));                                       \
+        const uint32_t ko_ = row_ * D + (((pos % CPR) ^ k_swz<D>(pos / CPR)) * 16u);                          \
         __builtin_amdgcn_global_load_lds((glb_ptr_t)(kb_ + ko_), (lds_ptr_t)(lk_ + u * 1024), 16, 0, 0);      \
         __builtin_amdgcn_global_load_lds((glb_ptr_t)(vb_ + v_lane + u * 1024), (lds_ptr_t)(lv_ + u * 1024), 16, 0, 0); \
       }                                                                                                       \

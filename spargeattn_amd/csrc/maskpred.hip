@@ -467,6 +467,265 @@ __global__ __launch_bounds__(256) void block_select_kernel(
 }
 
 // =============================================================================================
+// block_select, wavefront-per-row variant (nk <= 2048).
+// Phase 1 is the same score computation, two columns per lane at a time so that one broadcast LDS read of pooled Q
+// feeds four multiply-adds.  Phase 2 gives each of the four wavefronts its own rows and keeps a whole row in
+// registers (EPL = nkp / 64 columns per lane): no workgroup barrier, the stable descending sort is a bitonic network
+// whose short-distance steps are register-local and whose long-distance steps are lane exchanges.
+// dynamic LDS: R*D*8 (pooled Q as doubles) + R*nkp*4 (scores) + 4*nkp*4 (per-wave index list) + 4*64*8 (lane sums).
+// =============================================================================================
+template <int EPL, int K, int J>
+__device__ __forceinline__ void bitonic_step(uint32_t (&key)[EPL], int lane) {
+  constexpr int NKP = 64 * EPL;
+  // element v = lane * EPL + t; a step compares v with v ^ J inside blocks of size K (descending where (v & K) == 0)
+  if constexpr (J >= EPL) {
+    constexpr int DL = J / EPL;                                     // partner lane = lane ^ DL
+    const bool lower = (lane & DL) == 0;
+    const bool desc = (K >= NKP) ? true : ((lane & (K / EPL)) == 0);
+    const bool want_max = lower == desc;
+#pragma unroll
+    for (int t = 0; t < EPL; t++) {
+      const uint32_t o = (uint32_t)__shfl_xor((int)key[t], DL, SPG_WAVE);
+      const uint32_t mx = key[t] > o ? key[t] : o, mn = key[t] > o ? o : key[t];
+      key[t] = want_max ? mx : mn;
+    }
+  } else {
+#pragma unroll
+    for (int t = 0; t < EPL; t++) {
+      if ((t & J) == 0) {
+        const uint32_t a = key[t], b = key[t | J];
+        const uint32_t mx = a > b ? a : b, mn = a > b ? b : a;
+        if constexpr (K < EPL) {
+          const bool desc = (t & K) == 0;                           // compile-time
+          key[t] = desc ? mx : mn;
+          key[t | J] = desc ? mn : mx;
+        } else {
+          const bool desc = (K >= NKP) ? true : ((lane & (K / EPL)) == 0);
+          key[t] = desc ? mx : mn;
+          key[t | J] = desc ? mn : mx;
+        }
+      }
+    }
+  }
+}
+template <int EPL, int K, int J>
+__device__ __forceinline__ void bitonic_inner(uint32_t (&key)[EPL], int lane) {
+  bitonic_step<EPL, K, J>(key, lane);
+  if constexpr (J > 1) bitonic_inner<EPL, K, J / 2>(key, lane);
+}
+template <int EPL, int K>
+__device__ __forceinline__ void bitonic_sort_desc(uint32_t (&key)[EPL], int lane) {
+  bitonic_inner<EPL, K, K / 2>(key, lane);
+  if constexpr (K < 64 * EPL) bitonic_sort_desc<EPL, K * 2>(key, lane);
+}
+
+template <int D, int DT, int R, int EPL>
+__global__ __launch_bounds__(256) void block_select_wave_kernel(
+    const uint16_t *__restrict__ pool_q, const uint8_t *__restrict__ sim_q, const uint16_t *__restrict__ pool_k,
+    const uint8_t *__restrict__ sim_k, const float *__restrict__ topk, const float *__restrict__ cdfthr, int is_causal,
+    int sink, int32_t *__restrict__ lut, int32_t *__restrict__ valid, uint8_t *__restrict__ bmap, int H, int nq,
+    int nk) {
+  constexpr int NKP = 64 * EPL;
+  extern __shared__ __align__(16) unsigned char smem[];
+  double *s_pq = (double *)smem;                                              // [R][D]
+  float *s_scores = (float *)(smem + (size_t)R * D * 8);                      // [R][NKP]
+  int32_t *s_idx_all = (int32_t *)(smem + (size_t)R * D * 8 + (size_t)R * NKP * 4);   // [4][NKP]
+  double *s_lsum_all = (double *)(smem + (size_t)R * D * 8 + (size_t)R * NKP * 4 + 4 * (size_t)NKP * 4);   // [4][64]
+
+  const int i0 = blockIdx.x * R, bh = blockIdx.y, h = bh % H, tid = threadIdx.x;
+  const int rows = min(R, nq - i0);
+  for (int t = tid; t < R * D; t += 256) {
+    const int row = t / D;
+    s_pq[t] = row < rows ? (double)elem_to_f32<DT>(pool_q[((size_t)bh * nq + i0 + row) * D + (t % D)]) : 0.0;
+  }
+  __syncthreads();
+
+  const float sm_scale = (D == 64) ? 0.125f : 0.088388347648318447f;  // fp32(D^-0.5)
+  const uint16_t *pk_base = pool_k + (size_t)bh * nk * D;
+  const uint8_t *simk = sim_k + (size_t)bh * nk;
+
+  // ---- phase 1: scores, binary64 accumulation in the fixed order d = 0..D-1 (products of 16-bit floats are exact) ----
+  // columns at or beyond j_live are masked for every row of this workgroup: no arithmetic for them
+  const int j_live = is_causal ? min(nk, 2 * (i0 + rows)) : nk;
+  for (int jb = 0; jb < NKP; jb += 512) {
+    const int ja = jb + tid, jc = jb + 256 + tid;
+    const bool live_a = ja < j_live, live_c = jc < j_live;
+    double acc_a[R], acc_c[R];
+#pragma unroll
+    for (int row = 0; row < R; row++) { acc_a[row] = 0.0; acc_c[row] = 0.0; }
+    if (jb < j_live) {                                               // workgroup-uniform
+      const uint4 *krow_a = (const uint4 *)(pk_base + (size_t)(live_a ? ja : 0) * D);
+      const uint4 *krow_c = (const uint4 *)(pk_base + (size_t)(live_c ? jc : 0) * D);
+      const bool two = jb + 256 < j_live;                            // workgroup-uniform
+#pragma unroll 1
+      for (int cch = 0; cch < D / 8; cch++) {
+        const uint4 va = krow_a[cch];
+        const uint32_t wa[4] = {va.x, va.y, va.z, va.w};
+        double ka[8];
+#pragma unroll
+        for (int e = 0; e < 8; e++)
+          ka[e] = (double)elem_to_f32<DT>((uint16_t)((e & 1) ? (wa[e >> 1] >> 16) : (wa[e >> 1] & 0xffffu)));
+        if (two) {
+          const uint4 vc = krow_c[cch];
+          const uint32_t wc[4] = {vc.x, vc.y, vc.z, vc.w};
+          double kc[8];
+#pragma unroll
+          for (int e = 0; e < 8; e++)
+            kc[e] = (double)elem_to_f32<DT>((uint16_t)((e & 1) ? (wc[e >> 1] >> 16) : (wc[e >> 1] & 0xffffu)));
+#pragma unroll
+          for (int row = 0; row < R; row++) {
+            const double *q = s_pq + row * D + cch * 8;
+#pragma unroll
+            for (int e = 0; e < 8; e++) {
+              const double qe = q[e];
+              acc_a[row] = __builtin_fma(qe, ka[e], acc_a[row]);
+              acc_c[row] = __builtin_fma(qe, kc[e], acc_c[row]);
+            }
+          }
+        } else {
+#pragma unroll
+          for (int row = 0; row < R; row++) {
+            const double *q = s_pq + row * D + cch * 8;
+#pragma unroll
+            for (int e = 0; e < 8; e++) acc_a[row] = __builtin_fma(q[e], ka[e], acc_a[row]);
+          }
+        }
+      }
+    }
+    const bool dead_a = !live_a || simk[ja] == 0, dead_c = !live_c || simk[jc] == 0;
+#pragma unroll
+    for (int row = 0; row < R; row++) {
+      const float a1 = elem_to_f32<DT>(f64_to_elem<DT>(acc_a[row]));
+      float a2 = elem_to_f32<DT>(f64_to_elem<DT>((double)a1 * (double)sm_scale));
+      if (dead_a || (is_causal && ja >= 2 * (i0 + row + 1))) a2 = -INFINITY;
+      s_scores[(size_t)row * NKP + ja] = a2;
+      if (NKP > 256) {
+        const float c1 = elem_to_f32<DT>(f64_to_elem<DT>(acc_c[row]));
+        float c2 = elem_to_f32<DT>(f64_to_elem<DT>((double)c1 * (double)sm_scale));
+        if (dead_c || (is_causal && jc >= 2 * (i0 + row + 1))) c2 = -INFINITY;
+        s_scores[(size_t)row * NKP + jc] = c2;
+      }
+    }
+  }
+  __syncthreads();
+
+  // ---- phase 2: wavefront `wave` owns rows wave, wave + 4, ...; lane l holds columns l, l + 64, ... ----------------
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  int32_t *s_idx = s_idx_all + wave * NKP;
+  double *s_lsum = s_lsum_all + wave * 64;
+  for (int row = wave; row < rows; row += 4) {
+    const int i = i0 + row;
+    const int causal_lim = is_causal ? min(nk, 2 * (i + 1)) : nk;
+    const float *s_score = s_scores + (size_t)row * NKP;
+
+    float sc[EPL];
+    float lmax = -INFINITY;
+#pragma unroll
+    for (int t = 0; t < EPL; t++) {
+      sc[t] = s_score[t * 64 + lane];               // columns >= nk were written as -inf by phase 1
+      lmax = fmaxf(lmax, sc[t]);
+    }
+    const float mx = wave_max_f32(lmax);
+
+    // exp and the fixed summation tree: lane l adds e[l], e[l+64], ... in order, then an xor butterfly (32 .. 1)
+    double ev[EPL];
+    double part = 0.0;
+#pragma unroll
+    for (int t = 0; t < EPL; t++) {
+      ev[t] = (sc[t] == -INFINITY) ? 0.0 : cexp((double)sc[t] - (double)mx);
+      part = part + ev[t];
+    }
+#pragma unroll
+    for (int o = 32; o >= 1; o >>= 1) part = part + shfl_xor_f64(part, o);
+    const double total = part;
+
+    // probabilities -> sortable keys (value bits, then lower column first)
+    uint32_t okey[EPL], key[EPL];
+#pragma unroll
+    for (int t = 0; t < EPL; t++) {
+      const int j = t * 64 + lane;
+      double p = ev[t] / total;
+      if (!__builtin_isfinite(p)) p = 0.0;
+      const uint32_t bits = f64_to_elem<DT>(p);
+      okey[t] = j < nk ? ((bits << 16) | (0xffffu - (uint32_t)j)) : 0u;
+      key[t] = okey[t];
+    }
+    bitonic_sort_desc<EPL, 2>(key, lane);             // sorted position of key[t] is lane * EPL + t
+
+    // how many to keep
+    long long n;
+    if (topk != nullptr) {
+      const float t = topk[h] * (float)nk;            // binary32 product, truncated (utils.py:405)
+      n = (long long)t;
+    } else {
+      // cdf[v] = T(sum_{u<=v} p_sorted[u]);  n = #{v < nk : cdf[v] <= threshold}  (utils.py:398-403)
+      double lsum = 0.0;
+#pragma unroll
+      for (int t = 0; t < EPL; t++) lsum += (double)elem_to_f32<DT>((uint16_t)(key[t] >> 16));
+      s_lsum[lane] = lsum;
+      __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+      __builtin_amdgcn_wave_barrier();
+      double run = 0.0;
+      for (int u = 0; u < lane; u++) run += s_lsum[u];
+      const double thr = (double)cdfthr[h];
+      int cnt = 0;
+#pragma unroll
+      for (int t = 0; t < EPL; t++) {
+        run += (double)elem_to_f32<DT>((uint16_t)(key[t] >> 16));
+        const float cdfv = elem_to_f32<DT>(f64_to_elem<DT>(run));
+        if (lane * EPL + t < nk && (double)cdfv <= thr) cnt++;
+      }
+      n = wave_sum_i32(cnt);
+      __builtin_amdgcn_wave_barrier();
+    }
+    if (n <= 0) n = 1;                                // utils.py:289
+    uint32_t kth = 0u;
+    if (n < nk) {                                     // wavefront-uniform
+      const int pos = (int)n - 1, src = pos / EPL, tt = pos % EPL;
+      uint32_t mine = key[0];
+#pragma unroll
+      for (int t = 1; t < EPL; t++) mine = (tt == t) ? key[t] : mine;
+      kth = (uint32_t)__shfl((int)mine, src, SPG_WAVE);
+    }
+
+    // block map row, ascending index list, delta LUT
+    const bool row_forced = sim_q[(size_t)bh * nq + i] == 0;
+    const size_t row_off = ((size_t)bh * nq + i) * nk;
+    int base = 0;
+#pragma unroll
+    for (int t = 0; t < EPL; t++) {
+      const int j = t * 64 + lane;
+      bool f = false;
+      if (j < nk) {
+        f = row_forced || (okey[t] >= kth) || (simk[j] == 0);
+        if (j >= causal_lim) f = false;
+        if (sink && j == 0) f = true;
+        if (bmap != nullptr) bmap[row_off + j] = f ? 1 : 0;
+      }
+      const unsigned long long m = __ballot(f);
+      const int below = __builtin_amdgcn_mbcnt_hi((uint32_t)(m >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)m, 0));
+      if (f) s_idx[base + below] = j;
+      base += __builtin_popcountll(m);
+    }
+    __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+#pragma unroll
+    for (int t = 0; t < EPL; t++) {
+      const int pidx = t * 64 + lane;
+      if (pidx < nk) {
+        int v = 0;
+        if (pidx < base) v = s_idx[pidx] - (pidx ? s_idx[pidx - 1] : 0);
+        lut[row_off + pidx] = v;
+      }
+    }
+    if (lane == 0) valid[(size_t)bh * nq + i] = base;
+    __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+    __builtin_amdgcn_wave_barrier();                  // the index list is reused by this wavefront's next row
+  }
+}
+
+// =============================================================================================
 // user mask -> LUT
 // =============================================================================================
 template <int KIND>
@@ -580,6 +839,26 @@ static hipError_t launch_bs2(const void *pq, const uint8_t *sq, const void *pk, 
                              const float *cdf, int causal, int sink, int32_t *lut, int32_t *valid, uint8_t *bmap, int B,
                              int H, int nq, int nk, hipStream_t st) {
   const int nkp = next_pow2_ge(nk, 256);
+  if (nkp <= 2048) {
+    // a whole row fits the registers of one wavefront
+#define SPG_BSW(R_, EPL_)                                                                                       \
+    {                                                                                                           \
+      const size_t lds = (size_t)R_ * D * 8 + (size_t)R_ * nkp * 4 + 16 * (size_t)nkp + 4 * 64 * 8;             \
+      auto kern = block_select_wave_kernel<D, DT, R_, EPL_>;                                                    \
+      if (lds > 48 * 1024) {                                                                                    \
+        hipError_t e = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds); \
+        if (e != hipSuccess) return e;                                                                          \
+      }                                                                                                         \
+      kern<<<dim3((nq + R_ - 1) / R_, B * H), 256, lds, st>>>((const uint16_t *)pq, sq, (const uint16_t *)pk, sk, topk, \
+                                                              cdf, causal, sink, lut, valid, bmap, H, nq, nk);  \
+      return hipSuccess;                                                                                        \
+    }
+    if (nkp == 256) SPG_BSW(8, 4)
+    if (nkp == 512) SPG_BSW(8, 8)
+    if (nkp == 1024) SPG_BSW(8, 16)
+    SPG_BSW(4, 32)
+#undef SPG_BSW
+  }
   // rows per workgroup: reuse of the pooled-K reads against LDS footprint (scores are R*nkp floats)
   if (nkp <= 1024) return launch_bs3<D, DT, 8>(pq, sq, pk, sk, topk, cdf, causal, sink, lut, valid, bmap, B, H, nq, nk, nkp, st);
   if (nkp <= 4096) return launch_bs3<D, DT, 4>(pq, sq, pk, sk, topk, cdf, causal, sink, lut, valid, bmap, B, H, nq, nk, nkp, st);
