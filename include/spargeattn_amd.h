@@ -100,9 +100,15 @@ int spg_block_sparse_attn(const int8_t *q8, const int8_t *k8, const uint8_t *v8,
 
 /* ---- measurement comparator: dense FP16 flash attention on MFMA (no counterpart in the reference;
  * the "dense FP16 attention kernel built in the same run" the speed-up is quoted against).
- * q,k,v,out (B,H,N,D) fp16. */
-int spg_dense_attn_f16(const void *q, const void *k, const void *v, void *out, int B, int H, int N, int D,
+ * q,k,out (B,H,N,D) fp16; vt = V transposed per 64-key block, (B,H,ceil(N/64),D,64) fp16, zero-padded. */
+int spg_dense_attn_f16(const void *q, const void *k, const void *vt, void *out, int B, int H, int N, int D,
                        float sm_scale, int is_causal, void *stream);
+
+/* ---- self test (no counterpart in the reference): the INT8 quantisation and the cosine normalisation divide by
+ * a per-block / per-row value through a shared reciprocal; this entry point compares that division with the
+ * hardware's correctly rounded one for every finite fp16 and bf16 numerator against n_divisors pseudo-random
+ * divisors.  counts (device, 2 x uint64, zeroed by the caller): [0] += comparisons, [1] += mismatches. */
+int spg_selftest_division(unsigned long long *counts, int n_divisors, unsigned int seed, void *stream);
 
 #ifdef __cplusplus
 }

@@ -31,6 +31,7 @@ SIGNATURES = {
     "spg_v_quant_fp8": (_i, [_vp, _vp, _vp, _i, _i, _i, _i, _i, _vp]),
     "spg_block_sparse_attn": (_i, [_vp, _vp, _vp, _vp, _i, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _f, _i, _vp, _vp]),
     "spg_dense_attn_f16": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _f, _i, _vp]),
+    "spg_selftest_division": (_i, [_vp, _i, ctypes.c_uint, _vp]),
 }
 
 _lib = None
@@ -219,3 +220,10 @@ def dense_attn_f16(q, k, vt, sm_scale, is_causal=False, out=None):
     _check(load().spg_dense_attn_f16(_p(q), _p(k), _p(vt), _p(out), B, H, N, D, float(sm_scale),
                                      int(bool(is_causal)), _stream()))
     return out
+
+
+def selftest_division(n_divisors, seed=1):
+    """Returns (comparisons, mismatches) of the shared-reciprocal division against the hardware's IEEE division."""
+    counts = torch.zeros(2, dtype=torch.int64, device="cuda")
+    _check(load().spg_selftest_division(_p(counts), int(n_divisors), int(seed), _stream()))
+    return tuple(int(c) for c in counts.cpu())

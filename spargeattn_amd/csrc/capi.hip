@@ -102,6 +102,14 @@ int spg_map_to_lut(const void *mask, int mask_kind, int32_t *lut, int32_t *valid
   return check_launch(fn, spg::launch_map_to_lut(mask, mask_kind, lut, valid_block_num, B, H, nq, nk, (hipStream_t)stream));
 }
 
+int spg_selftest_division(unsigned long long *counts, int n_divisors, unsigned int seed, void *stream) {
+  const char *fn = "spg_selftest_division";
+  if (n_divisors <= 0 || n_divisors > (1 << 22)) return fail(SPG_ERR_INVALID, "%s: n_divisors must be in [1, 2^22]", fn);
+  SPG_NONNULL(fn, counts);
+  spg::launch_div_selftest(counts, n_divisors, seed, (hipStream_t)stream);
+  return check_launch(fn, hipSuccess);
+}
+
 int spg_v_quant_fp8(const void *v, uint8_t *v8, float *v_scale, int B, int H, int N, int D, int dtype, void *stream) {
   const char *fn = "spg_v_quant_fp8";
   SPG_TRY(check_shape(fn, B, H, N, D));

@@ -56,10 +56,22 @@ template <> __device__ __forceinline__ uint16_t f32_to_elem<0>(float x) {
   return __builtin_bit_cast(uint16_t, h);
 }
 template <> __device__ __forceinline__ uint16_t f32_to_elem<1>(float x) {
-  const uint32_t u = __builtin_bit_cast(uint32_t, x);
-  const uint32_t rounded = (u + 0x7fffu + ((u >> 16) & 1u)) >> 16;
-  const uint32_t quiet = (u >> 16) | 0x40u;
-  return (uint16_t)(((u & 0x7fffffffu) > 0x7f800000u) ? quiet : rounded);   // select, no branch
+  return __builtin_bit_cast(uint16_t, (__bf16)x);   // v_cvt_pk_bf16_f32: round to nearest even in hardware
+}
+
+// Round two binary32 values to the 16-bit element type and widen them again (one packed conversion for bfloat16).
+template <int DT> __device__ __forceinline__ void round2_through_elem(float &a, float &b);
+template <> __device__ __forceinline__ void round2_through_elem<0>(float &a, float &b) {
+  a = (float)(_Float16)a;
+  b = (float)(_Float16)b;
+}
+template <> __device__ __forceinline__ void round2_through_elem<1>(float &a, float &b) {
+  typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+  typedef float f32x2 __attribute__((ext_vector_type(2)));
+  const f32x2 v = {a, b};
+  const uint32_t u = __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2));
+  a = __builtin_bit_cast(float, u << 16);
+  b = __builtin_bit_cast(float, u & 0xffff0000u);
 }
 
 // ---------------------------------------------------------------------------------------------

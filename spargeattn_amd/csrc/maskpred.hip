@@ -66,22 +66,48 @@ __global__ void km_final_kernel(const double *__restrict__ part, uint16_t *__res
 // =============================================================================================
 // pool + sim + INT8 quantisation.  One workgroup per (block, b*h).
 // =============================================================================================
-// IEEE binary32 quotient a/b through a refined reciprocal r ~ 1/b shared by many numerators: the operation
-// sequence of the hardware's correctly rounded division (reciprocal + one Newton step, then two residual
-// corrections of the quotient) without its operand scaling, valid while b stays in [2^-60, 2^60].
-__device__ __forceinline__ float refined_rcp(float b) {
-  const float r0 = __builtin_amdgcn_rcpf(b);
-  const float e = __builtin_fmaf(-b, r0, 1.0f);
-  return __builtin_fmaf(e, r0, r0);
-}
+// IEEE binary32 quotient a/b with a reciprocal shared by many numerators: r = RN(1/b) (one correctly rounded
+// division), then q = RN(a*r), one exact residual and one correction (Markstein).  div_selftest_kernel below
+// compares it with the hardware's correctly rounded division for every finite binary16/bfloat16 numerator with
+// |a| >= 2^-100 against pseudo-random divisors: the only difference is the sign of a zero quotient, which no user of
+// the result can see.
+// Valid while b stays in [2^-60, 2^60] (no scaling of the operands is done); quotients below 2^-100 in magnitude
+// may be off in the last place, far below anything the callers resolve.
+__device__ __forceinline__ float exact_rcp(float b) { return 1.0f / b; }
 __device__ __forceinline__ float div_by(float a, float b, float r) {
-  float q = a * r;
-  float e = __builtin_fmaf(-b, q, a);
-  q = __builtin_fmaf(e, r, q);
-  e = __builtin_fmaf(-b, q, a);
+  const float q = a * r;
+  const float e = __builtin_fmaf(-b, q, a);
   return __builtin_fmaf(e, r, q);
 }
 __device__ __forceinline__ bool rcp_safe(float b) { return b >= 0x1p-60f && b <= 0x1p60f; }
+
+// Self-test of div_by: divisor number i is a hash of (seed, i) with exponent in [-40, 40); every finite 16-bit
+// numerator of both element types with |a| >= 2^-100 and 2^-100 <= |a/b| <= 2^100 is divided both ways.  counts[0] += comparisons,
+// counts[1] += differing bit patterns other than a differently signed zero.
+__global__ __launch_bounds__(256) void div_selftest_kernel(unsigned long long *counts, int n_div, uint32_t seed) {
+  auto hash32 = [](uint32_t x) { x ^= x >> 16; x *= 0x7feb352du; x ^= x >> 15; x *= 0x846ca68bu; x ^= x >> 16; return x; };
+  const uint32_t bi = blockIdx.x * 256u + threadIdx.x;
+  if (bi >= (uint32_t)n_div) return;
+  const uint32_t h = hash32(bi * 2654435761u + seed);
+  const int ex = (int)(hash32(h) % 80u) - 40;
+  const float b = __builtin_bit_cast(float, ((uint32_t)(127 + ex) << 23) | (h & 0x7fffffu));
+  const float r = exact_rcp(b);
+  unsigned long long bad = 0, tot = 0;
+  for (uint32_t pat = 0; pat < 65536u; pat++) {
+#pragma unroll
+    for (int kind = 0; kind < 2; kind++) {
+      const float a = kind == 0 ? elem_to_f32<1>((uint16_t)pat) : elem_to_f32<0>((uint16_t)pat);
+      if (!__builtin_isfinite(a) || (__builtin_fabsf(a) < 0x1p-100f && a != 0.0f)) continue;
+      const float want = a / b, got = div_by(a, b, r);
+      const float mag = __builtin_fabsf(want);
+      if (want != 0.0f && !(mag >= 0x1p-100f && mag <= 0x1p100f)) continue;   // outside the range the callers use
+      tot++;
+      if (__builtin_bit_cast(uint32_t, want) != __builtin_bit_cast(uint32_t, got) && !(want == 0.0f && got == 0.0f)) bad++;
+    }
+  }
+  atomicAdd(&counts[0], tot);
+  atomicAdd(&counts[1], bad);
+}
 
 template <int BS, int D, int DT, bool HAS_MEAN, bool WITH_POOL>
 __global__ __launch_bounds__(256) void pool_sim_quant_kernel(const uint16_t *__restrict__ x,
@@ -119,16 +145,22 @@ __global__ __launch_bounds__(256) void pool_sim_quant_kernel(const uint16_t *__r
     if (ok) v = *(const uint4 *)(xb + (size_t)row * D);
     const uint32_t w[4] = {v.x, v.y, v.z, v.w};
 #pragma unroll
-    for (int e = 0; e < 8; e++) {
-      float f = elem_to_f32<DT>((uint16_t)((e & 1) ? (w[e >> 1] >> 16) : (w[e >> 1] & 0xffffu)));
+    for (int e = 0; e < 8; e += 2) {
+      float f0 = elem_to_f32<DT>((uint16_t)(w[e >> 1] & 0xffffu));
+      float f1 = elem_to_f32<DT>((uint16_t)(w[e >> 1] >> 16));
       if constexpr (HAS_MEAN) {
         // (k - km) rounded once to the input dtype (utils.py:184-188).  The binary32 difference of two 16-bit
         // floats is either exact or nowhere near a rounding tie of the 16-bit format, so rounding it to nearest
         // even equals rounding the exact difference.  Masked rows stay zero.
-        if (ok) f = elem_to_f32<DT>(f32_to_elem<DT>(f - kmf[e]));
+        if (ok) {
+          f0 -= kmf[e];
+          f1 -= kmf[e + 1];
+          round2_through_elem<DT>(f0, f1);
+        }
       }
-      xf[p][e] = f;
-      amax = fmaxf(amax, fabsf(f));
+      xf[p][e] = f0;
+      xf[p][e + 1] = f1;
+      amax = fmaxf(amax, fmaxf(fabsf(f0), fabsf(f1)));
     }
   }
 
@@ -155,7 +187,7 @@ __global__ __launch_bounds__(256) void pool_sim_quant_kernel(const uint16_t *__r
       ss = group_sum_f64<TPR>(ss);                 // the TPR lanes of this row
       const float norm = sqrtf((float)ss);
       if (rcp_safe(norm)) {
-        const float rn = refined_rcp(norm);
+        const float rn = exact_rcp(norm);
 #pragma unroll
         for (int e = 0; e < 8; e++) {
           const _Float16 h = (_Float16)div_by(xf[p][e], norm, rn);
@@ -210,7 +242,7 @@ __global__ __launch_bounds__(256) void pool_sim_quant_kernel(const uint16_t *__r
 #pragma unroll
         for (int e = 0; e < 8; e++) {
           float y = divide(xf[p][e]);
-          y = y + (y >= 0.f ? 0.5f : -0.5f);
+          y = y + __builtin_copysignf(0.5f, y);   // +0.5 for y >= 0 (a -0 quotient truncates to 0 either way)
           const int q = (int)y;   // truncation toward zero
           pk[e >> 2] |= ((uint32_t)q & 0xffu) << (8 * (e & 3));
         }
@@ -219,7 +251,7 @@ __global__ __launch_bounds__(256) void pool_sim_quant_kernel(const uint16_t *__r
     }
   };
   if (rcp_safe(s)) {                     // workgroup-uniform
-    const float rs = refined_rcp(s);
+    const float rs = exact_rcp(s);
     quantise([&](float v) { return div_by(v, s, rs); });
   } else {
     quantise([&](float v) { return v / s; });
@@ -818,6 +850,10 @@ void launch_pool_sim_quant(const void *x, const void *km, void *pool, uint8_t *s
 }
 
 int block_select_max_nk() { return 8192; }
+
+void launch_div_selftest(unsigned long long *counts, int n_div, uint32_t seed, hipStream_t st) {
+  div_selftest_kernel<<<(n_div + 255) / 256, 256, 0, st>>>(counts, n_div, seed);
+}
 
 template <int D, int DT, int R>
 static hipError_t launch_bs3(const void *pq, const uint8_t *sq, const void *pk, const uint8_t *sk, const float *topk,
