@@ -98,6 +98,22 @@ int spg_block_sparse_attn(const int8_t *q8, const int8_t *k8, const uint8_t *v8,
                           int B, int H, int N, int D, float sm_scale, int is_causal, int32_t *pv_count,
                           void *stream);
 
+/* ---- SageAttention1-style variant: INT8 QK^T, FP16 PV.
+ * Replaces qk_int8_sv_f16_accum_f16_block_sparse_attn_inst_buf_with_pv_threshold (csrc/qattn/attn_cuda.h:32-45,
+ * kernel csrc/qattn/qk_int_sv_f16_cuda_sm80.cuh:42-671) as called by spas_sage_attn_meansim[_topk]_cuda
+ * (spas_sage_attn/core.py:235-319): P is rounded to fp16, the denominator sums the rounded P, the output is O / d
+ * with no V scale, is_causal masks at token level.  PV is accumulated in fp32 throughout (the reference rounds each
+ * 64-key partial product to fp16 first).
+ * spg_v_tiles_f16 prepares the V operand: v (B,H,N,D) fp16|bf16 -> vt (B,H,ceil(N/64),D,64) fp16, the V^T of each
+ * 64-key block (bf16 is rounded to fp16 as core.py:247 does), 8-key chunks of a row stored at slot chunk ^ (d & 7),
+ * zero beyond N.  It takes the place of the kernel's transposing shared-memory reads (ldmatrix.trans). */
+int spg_v_tiles_f16(const void *v, void *vt, int B, int H, int N, int D, int dtype, void *stream);
+int spg_block_sparse_attn_f16v(const int8_t *q8, const int8_t *k8, const void *vt, void *out, int out_dtype,
+                               const int32_t *lut, const int32_t *valid_block_num, const float *pvthreshd,
+                               const float *q_scale, const float *k_scale,
+                               int B, int H, int N, int D, float sm_scale, int is_causal, int32_t *pv_count,
+                               void *stream);
+
 /* ---- measurement comparator: dense FP16 flash attention on MFMA (no counterpart in the reference;
  * the "dense FP16 attention kernel built in the same run" the speed-up is quoted against).
  * q,k,out (B,H,N,D) fp16; vt = V transposed per 64-key block, (B,H,ceil(N/64),D,64) fp16, zero-padded. */

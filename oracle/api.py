@@ -1,8 +1,9 @@
 """End-to-end oracle of the two operator entry points.  Test infrastructure only.
 
-``spas_sage2_attn_meansim_topk`` follows spas_sage_attn/core.py:105-169 and
+``spas_sage2_attn_meansim_topk`` follows spas_sage_attn/core.py:105-169,
 ``block_sparse_sage2_attn`` follows spas_sage_attn/core.py:171-233 (non-sm90
-branch: BLKQ = 128, BLKK = 64), returning every intermediate tensor so that a
+branch: BLKQ = 128, BLKK = 64) and ``spas_sage_attn_meansim_topk`` follows
+spas_sage_attn/core.py:235-319, returning every intermediate tensor so that a
 test can compare stage by stage.  Inputs are numpy float32 arrays in HND layout
 whose values are representable in ``dtype`` (bf16 or fp16).
 """
@@ -70,6 +71,27 @@ def spas_sage2_attn_meansim_topk(q, k, v, dtype, is_causal=False, scale=None, si
     if stop_after_mask:
         return res
     return _common_tail(res, q, v, dtype, pvthreshd, scale, kernel_causal)
+
+
+def spas_sage_attn_meansim_topk(q, k, v, dtype, is_causal=False, scale=None, simthreshd1=-0.1, cdfthreshd=None,
+                                topk=0.5, pvthreshd=50, attention_sink=False):
+    """core.py:278-319 (and 235-276 with cdfthreshd): the mask prediction of the Sage2 operator, then the INT8-QK /
+    FP16-PV kernel on fp16(v) with the token-level causal flag (core.py:308-310)."""
+    res = spas_sage2_attn_meansim_topk(q, k, v, dtype, is_causal=is_causal, scale=scale, simthreshd1=simthreshd1,
+                                       cdfthreshd=cdfthreshd, topk=topk, attention_sink=attention_sink,
+                                       stop_after_mask=True)
+    q = np.asarray(q, dtype=F32)
+    b, h, n, d = q.shape
+    nk = (n + 63) // 64
+    v16 = np.zeros((b, h, nk * 64, d), dtype=F32)
+    v16[:, :, :n] = vq.to_fp16(v)
+    res["v16"] = v16
+    sm_scale = (1.0 / d ** 0.5) if scale is None else scale
+    out, written, pvc = at.block_sparse_attention(
+        res["q8"], res["k8"], v16, res["lut"], res["valid"], hyperparameter(h, pvthreshd), res["q_scale"],
+        res["k_scale"], None, sm_scale, dtype, is_causal=bool(is_causal), return_pv_count=True, pv="f16")
+    res["out"], res["written"], res["pv_count"] = out, written, pvc
+    return res
 
 
 def block_sparse_sage2_attn(q, k, v, mask_id, dtype, scale=None, pvthreshd=50, kernel_causal=False):

@@ -47,18 +47,29 @@ def _fma(a, b, c):
 
 
 def block_sparse_attention(q8, k8, v8, lut, valid, pvthreshd, q_scale, k_scale, v_scale,
-                           sm_scale, out_dtype, is_causal=False, return_pv_count=False):
+                           sm_scale, out_dtype, is_causal=False, return_pv_count=False, pv="fp8"):
     """q8,k8 int8 (B,H,N,D); v8 e4m3 codes uint8 (B,H,Npad,D); lut/valid int32.
 
     Returns (out float32 (B,H,N,D) holding out_dtype values, written (B,H,nq) bool[, pv_count (B,H,nq)]).
     Row blocks with valid == 0 are left untouched (zeros here; sm89.cuh:232-235).
+
+    ``pv="f16"`` restates the SageAttention1 kernel instead (qk_int_sv_f16_cuda_sm80.cuh:42-671 instantiated with
+    per-block quantisation, per-block PV threshold and the row sum on the tensor cores, sm80.cuh:690): ``v8`` then holds
+    fp16 VALUES (float array, (B,H,Npad,D), zero beyond N), ``v_scale`` is ignored, P has no exponent offset and is
+    rounded to fp16 (RS_32_to_16, attn_utils.cuh:563-580), the denominator sums the ROUNDED P in binary32
+    (accumulate_d on the tensor-core path, attn_utils.cuh:599-626) and the output is O / d.  The PV product is
+    accumulated in binary32 here; the reference accumulates the four 16-key steps of a block in fp16 before adding
+    the block to its binary32 accumulator (compute_fp16_sv_permuted_inst_buf, attn_utils.cuh:683-751) - parity
+    unpinned for that rounding, the comparison is by tolerance.
     """
+    assert pv in ("fp8", "f16")
     q8 = np.asarray(q8)
     k8 = np.asarray(k8)
     b_, h_, n, d_ = q8.shape
     nkv = k8.shape[2]
     nq = (n + CTA_Q - 1) // CTA_Q
-    vf = e4m3fn_to_f32(v8)
+    vf = e4m3fn_to_f32(v8) if pv == "fp8" else np.asarray(v8, dtype=F32)
+    offset = S_FP8_OFFSET if pv == "fp8" else F32(0.0)
     c = F32(F32(sm_scale) * LOG2E)
     out = np.zeros((b_, h_, n, d_), dtype=F32)
     written = np.zeros((b_, h_, nq), dtype=bool)
@@ -101,7 +112,7 @@ def block_sparse_attention(q8, k8, v8, lut, valid, pvthreshd, q_scale, k_scale, 
                         m = m_new
                         if not (F32(delta + thr) > 0):
                             continue
-                        neg_m = (-m + S_FP8_OFFSET).astype(F32)
+                        neg_m = (-m + offset).astype(F32)
                         p = _exp2(_fma(s, a, neg_m[:, None]))
                     else:
                         sf = (s * dq).astype(F32)
@@ -116,14 +127,20 @@ def block_sparse_attention(q8, k8, v8, lut, valid, pvthreshd, q_scale, k_scale, 
                         dsum = (dsum * o_scale).astype(F32)
                         o = (o * o_scale[:, None]).astype(F32)
                         m = m_new
-                        neg_m = (-m + S_FP8_OFFSET).astype(F32)
+                        neg_m = (-m + offset).astype(F32)
                         p = _exp2(_fma(sf, c, neg_m[:, None]))
                     cnt += 1
-                    dsum = (dsum + p.sum(axis=1, dtype=F32)).astype(F32)
-                    p8 = e4m3fn_to_f32(f32_to_e4m3fn(p))
+                    if pv == "fp8":
+                        dsum = (dsum + p.sum(axis=1, dtype=F32)).astype(F32)
+                        p8 = e4m3fn_to_f32(f32_to_e4m3fn(p))
+                    else:
+                        p8 = round_to(p.astype(np.float64), "fp16").astype(F32)
+                        dsum = (dsum + p8.sum(axis=1, dtype=F32)).astype(F32)
                     o = (o + (p8 @ vb).astype(F32)).astype(F32)
                 pv_count[b, h, i] = cnt
-                res = (o / dsum[:, None]).astype(F32) * np.asarray(v_scale[b, h], dtype=F32)[None, :]
+                res = (o / dsum[:, None]).astype(F32)
+                if pv == "fp8":
+                    res = res * np.asarray(v_scale[b, h], dtype=F32)[None, :]
                 out[b, h, r0:r0 + rows] = round_to(res[:rows].astype(np.float64), out_dtype)
     if return_pv_count:
         return out, written, pv_count

@@ -30,6 +30,8 @@ SIGNATURES = {
     "spg_map_to_lut": (_i, [_vp, _i, _vp, _vp, _i, _i, _i, _i, _vp]),
     "spg_v_quant_fp8": (_i, [_vp, _vp, _vp, _i, _i, _i, _i, _i, _vp]),
     "spg_block_sparse_attn": (_i, [_vp, _vp, _vp, _vp, _i, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _f, _i, _vp, _vp]),
+    "spg_v_tiles_f16": (_i, [_vp, _vp, _i, _i, _i, _i, _i, _vp]),
+    "spg_block_sparse_attn_f16v": (_i, [_vp] * 4 + [_i] + [_vp] * 5 + [_i] * 4 + [_f, _i, _vp, _vp]),
     "spg_dense_attn_f16": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _f, _i, _vp]),
     "spg_selftest_division": (_i, [_vp, _i, ctypes.c_uint, _vp]),
 }
@@ -198,6 +200,37 @@ def block_sparse_attn(q8, k8, v8, out, lut, valid, pvthreshd, q_scale, k_scale, 
     _check(load().spg_block_sparse_attn(_p(q8), _p(k8), _p(v8), _p(out), _dt(out), _p(lut), _p(valid), _p(pvthreshd),
                                         _p(q_scale), _p(k_scale), _p(v_scale), B, H, N, D, float(sm_scale),
                                         int(bool(is_causal)), _p(pvc), _stream()))
+    return pvc
+
+
+def v_tiles_f16_swizzled(v):
+    """v (B,H,N,D) fp16/bf16 -> (B,H,nk,D,64) fp16 V^T tiles, chunk-swizzled, the operand of block_sparse_attn_f16v."""
+    _dev(v)
+    B, H, N, D = v.shape
+    nk = (N + 63) // 64
+    vt = torch.empty((B, H, nk, D, 64), dtype=torch.float16, device=v.device)
+    _check(load().spg_v_tiles_f16(_p(v), _p(vt), B, H, N, D, _dt(v), _stream()))
+    return vt
+
+
+def v_tiles_f16_to_natural(vt):
+    """(B,H,nk,D,64) swizzled fp16 tiles -> (B,H,nk*64,D) in natural key order."""
+    B, H, nk, D, _ = vt.shape
+    d = torch.arange(D, device=vt.device)
+    idx = torch.arange(8, device=vt.device)[None, :] ^ (d & 7)[:, None]      # chunk kc sits at slot kc ^ (d & 7)
+    t = vt.view(B, H, nk, D, 8, 8)
+    nat = torch.gather(t, 4, idx.view(1, 1, 1, D, 8, 1).expand(B, H, nk, D, 8, 8))
+    return nat.reshape(B, H, nk, D, 64).permute(0, 1, 2, 4, 3).reshape(B, H, nk * 64, D)
+
+
+def block_sparse_attn_f16v(q8, k8, vt, out, lut, valid, pvthreshd, q_scale, k_scale, sm_scale, is_causal=False,
+                           return_pv_count=False):
+    _dev(q8, k8, vt, out, lut, valid, pvthreshd, q_scale, k_scale)
+    B, H, N, D = q8.shape
+    pvc = torch.zeros((B, H, (N + 127) // 128), dtype=torch.int32, device=q8.device) if return_pv_count else None
+    _check(load().spg_block_sparse_attn_f16v(_p(q8), _p(k8), _p(vt), _p(out), _dt(out), _p(lut), _p(valid),
+                                             _p(pvthreshd), _p(q_scale), _p(k_scale), B, H, N, D, float(sm_scale),
+                                             int(bool(is_causal)), _p(pvc), _stream()))
     return pvc
 
 

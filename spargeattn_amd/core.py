@@ -3,6 +3,8 @@
     spas_sage2_attn_meansim_topk_cuda   spas_sage_attn/core.py:105-169
     spas_sage2_attn_meansim_cuda        spas_sage_attn/core.py:39-103   (CDF selection)
     block_sparse_sage2_attn_cuda        spas_sage_attn/core.py:171-233
+    spas_sage_attn_meansim_cuda         spas_sage_attn/core.py:235-276  (INT8 QK^T, FP16 PV, CDF selection)
+    spas_sage_attn_meansim_topk_cuda    spas_sage_attn/core.py:278-319  (INT8 QK^T, FP16 PV, top-k selection)
 
 Same names, argument order, defaults and return values.  The ``_cuda`` suffix is kept so that
 callers need no change; everything runs as HIP kernels for gfx950.  As in the reference,
@@ -88,6 +90,51 @@ def _meansim(q, k, v, is_causal, scale, smooth_k, simthreshd1, cdfthreshd, topk,
         attention_sink=attention_sink, BLKQ=128, BLKK=64)
     o, _ = _attention(q, k, v, q_int8, q_scale, k_int8, k_scale, lut, valid_block_num, scale, pvthreshd, kernel_causal)
     return _finish(o, tensor_layout, return_sparsity, valid_block_num, lut, causal_denominator=is_causal is not False)
+
+
+def _meansim_sage1(q, k, v, is_causal, scale, smooth_k, simthreshd1, cdfthreshd, topk, pvthreshd, attention_sink,
+                   tensor_layout, return_sparsity):
+    """INT8 QK^T / FP16 PV path (spas_sage_attn/core.py:235-319): fp16 V, token-level causal masking in the kernel,
+    sparsity reported against the full grid unless is_causal."""
+    q, k, v = _prologue(q, k, v, tensor_layout)
+    if not smooth_k:
+        raise NameError("name 'km' is not defined")           # as the reference (core.py:249-252)
+    _mark("km")
+    km = _lib.km_mean(k)
+    _mark("maskpred")
+    lut, valid_block_num, q_int8, q_scale, k_int8, k_scale = get_block_map_meansim_fuse_quant(
+        q, k, km, is_causal=is_causal, simthreshd1=simthreshd1, cdfthreshd=cdfthreshd, topk=topk, return_lut=True,
+        attention_sink=attention_sink)
+    headdim = q.size(-1)
+    if scale is None:
+        scale = 1.0 / (headdim ** 0.5)
+    assert headdim in [64, 128], "headdim should be in [64, 128]. For other headdim, you can use padding and specify the softmax scale."
+    pvthreshd = hyperparameter_check(pvthreshd, q.size(-3), q.device)
+    o = torch.empty_like(q)
+    _mark("vquant")
+    vt = _lib.v_tiles_f16_swizzled(v)
+    _mark("attn")
+    _lib.block_sparse_attn_f16v(q_int8, k_int8, vt, o, lut, valid_block_num, pvthreshd, q_scale, k_scale, scale,
+                                is_causal=bool(is_causal))
+    _mark("end")
+    return _finish(o, tensor_layout, return_sparsity, valid_block_num, lut, causal_denominator=is_causal is not False)
+
+
+@torch.compiler.disable
+def spas_sage_attn_meansim_cuda(q, k, v, attn_mask=None, dropout_p=0.0, is_causal=False, scale=None, smooth_k=True,
+                                simthreshd1=0.6, cdfthreshd=0.98, pvthreshd=50, attention_sink=False,
+                                tensor_layout="HND", output_dtype=torch.float16, return_sparsity=False):
+    return _meansim_sage1(q, k, v, is_causal, scale, smooth_k, simthreshd1, cdfthreshd, None, pvthreshd,
+                          attention_sink, tensor_layout, return_sparsity)
+
+
+@torch.compiler.disable
+def spas_sage_attn_meansim_topk_cuda(q, k, v, attn_mask=None, dropout_p=0.0, is_causal=False, scale=None,
+                                     smooth_k=True, simthreshd1=-0.1, cdfthreshd=None, topk=0.5, pvthreshd=50,
+                                     attention_sink=False, tensor_layout="HND", output_dtype=torch.float16,
+                                     return_sparsity=False):
+    return _meansim_sage1(q, k, v, is_causal, scale, smooth_k, simthreshd1, cdfthreshd, topk, pvthreshd,
+                          attention_sink, tensor_layout, return_sparsity)
 
 
 @torch.compiler.disable

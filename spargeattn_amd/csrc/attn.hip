@@ -76,16 +76,25 @@ __device__ __forceinline__ uint32_t k_swz(uint32_t row) {
 }
 __device__ __forceinline__ int v_swz(int row) { return (row >> 1) & 3; }
 
-template <int D, int ODT>
-__global__ __launch_bounds__(256, 3) void block_sparse_attn_kernel(const AttnParams p) {
+// PV16 = false: V^T tiles are e4m3 (64 bytes per channel row), P is packed to e4m3 with the +8.807 exponent offset and
+//               the denominator sums the un-rounded P (the SageAttention2 kernel, sm89.cuh).
+// PV16 = true:  V^T tiles are fp16 (128 bytes per channel row, 16-byte chunks swizzled by slot = chunk ^ (d & 7)), P is
+//               rounded to fp16 and the denominator sums the ROUNDED P (the SageAttention1 kernel with the row sum on
+//               the matrix unit, qk_int_sv_f16_cuda_sm80.cuh:339-368, attn_utils.cuh:599-626).  The PV product is
+//               accumulated in fp32; the reference accumulates each 64-key block in fp16 before adding it to its fp32
+//               accumulator (attn_utils.cuh:683-751), a rounding this kernel does not reproduce.
+template <int D, int ODT, bool PV16>
+__global__ __launch_bounds__(256, PV16 ? 2 : 3) void block_sparse_attn_kernel(const AttnParams p) {
   constexpr int KS = D / 32;        // k-steps of the int8 MFMA
   constexpr int NDT = D / 32;       // 32-channel output tiles
-  constexpr int TILE = 64 * D;      // bytes of one K tile = bytes of one V^T tile
+  constexpr int TILE = 64 * D;      // bytes of one K tile
+  constexpr int VTILE = PV16 ? 2 * TILE : TILE;   // bytes of one V^T tile
   constexpr int CPR = D / 16;       // 16-byte chunks per K row
-  constexpr int WL = D / 64;        // global_load_lds instructions per wave per tile (TILE / 1024 / 4)
+  constexpr int WL = D / 64;        // global_load_lds instructions per wave per K tile (TILE / 1024 / 4)
+  constexpr int WLV = VTILE / 4096; // ... per V^T tile
   constexpr int NBUF = 3;
   // LDS: K ring [NBUF][TILE] | V^T ring [NBUF][TILE] | votes
-  __shared__ __align__(1024) unsigned char smem[2 * NBUF * TILE];
+  __shared__ __align__(1024) unsigned char smem[NBUF * (TILE + VTILE)];
   __shared__ int sVote[2][4];
   unsigned char *const sKr = smem;
   unsigned char *const sVr = smem + NBUF * TILE;
@@ -117,7 +126,7 @@ __global__ __launch_bounds__(256, 3) void block_sparse_attn_kernel(const AttnPar
   }
 
   const int8_t *kbase = p.k8 + (size_t)bh * N * D;
-  const uint8_t *vbase = p.v8 + (size_t)bh * p.nk * (size_t)TILE;
+  const uint8_t *vbase = p.v8 + (size_t)bh * p.nk * (size_t)VTILE;
   // LUT and K scales are read through the constant address space: uniform addresses become scalar loads (SMEM),
   // which never touch the vector-memory counter the tile ring is synchronised with.
   typedef const __attribute__((address_space(4))) int32_t *c_i32_t;
@@ -138,8 +147,8 @@ __global__ __launch_bounds__(256, 3) void block_sparse_attn_kernel(const AttnPar
   uint32_t lane_ = threadIdx.x & 63u;                                                                         \
   asm volatile("" : "+v"(lane_));                                                                             \
   const uint32_t pos0 = (uint32_t)(WL * 64 * wave) + lane_;                                                   \
-  const uint32_t v_lane = pos0 * 16u;                                                                         \
-  const uint32_t k_lane = v_lane ^ (k_swz<D>(pos0 / CPR) * 16u);   /* row * D + (slot ^ swz) * 16 */
+  const uint32_t v_lane = ((uint32_t)(WLV * 64 * wave) + lane_) * 16u;                                        \
+  const uint32_t k_lane = (pos0 * 16u) ^ (k_swz<D>(pos0 / CPR) * 16u);   /* row * D + (slot ^ swz) * 16 */
   const int last_partial_blk = (N % 64) ? p.nk - 1 : -1;   // the only block with rows beyond N
   typedef __attribute__((address_space(3))) void *lds_ptr_t;
   typedef const __attribute__((address_space(1))) void *glb_ptr_t;
@@ -147,15 +156,19 @@ __global__ __launch_bounds__(256, 3) void block_sparse_attn_kernel(const AttnPar
   {                                                                                                           \
     SPG_LANE_OFFSETS()                                                                                        \
     const int8_t *kb_ = kbase + (size_t)(BLK) * TILE;                                                         \
-    const uint8_t *vb_ = vbase + (size_t)(BLK) * TILE;                                                        \
+    const uint8_t *vb_ = vbase + (size_t)(BLK) * VTILE;                                                       \
     unsigned char *lk_ = sKr + (BUFOFF) + WL * wave * 1024;                                                   \
-    unsigned char *lv_ = sVr + (BUFOFF) + WL * wave * 1024;                                                   \
+    unsigned char *lv_ = sVr + (PV16 ? 2 * (BUFOFF) : (BUFOFF)) + WLV * wave * 1024;                          \
     if ((BLK) != last_partial_blk) {                                                                          \
       __builtin_amdgcn_global_load_lds((glb_ptr_t)(kb_ + k_lane), (lds_ptr_t)lk_, 16, 0, 0);                  \
       __builtin_amdgcn_global_load_lds((glb_ptr_t)(vb_ + v_lane), (lds_ptr_t)lv_, 16, 0, 0);                  \
-      if constexpr (WL == 2) {                                                                                \
+      if constexpr (WL == 2)                                                                                  \
         __builtin_amdgcn_global_load_lds((glb_ptr_t)(kb_ + k_lane), (lds_ptr_t)lk_, 16, 1024, 0);             \
+      if constexpr (WLV >= 2)                                                                                 \
         __builtin_amdgcn_global_load_lds((glb_ptr_t)(vb_ + v_lane), (lds_ptr_t)lv_, 16, 1024, 0);             \
+      if constexpr (WLV == 4) {                                                                               \
+        __builtin_amdgcn_global_load_lds((glb_ptr_t)(vb_ + v_lane), (lds_ptr_t)lv_, 16, 2048, 0);             \
+        __builtin_amdgcn_global_load_lds((glb_ptr_t)(vb_ + v_lane), (lds_ptr_t)lv_, 16, 3072, 0);             \
       }                                                                                                       \
     } else {                                                                                                  \
       /* rows beyond N are clamped to row N-1: their scores are masked, their V rows are zero */              \
@@ -165,8 +178,9 @@ __global__ __launch_bounds__(256, 3) void block_sparse_attn_kernel(const AttnPar
         const uint32_t row_ = min(pos / CPR, (uint32_t)(rows_ok_ - 1));                                       \
         const uint32_t ko_ = row_ * D + (((pos % CPR) ^ k_swz<D>(pos / CPR)) * 16u);                          \
         __builtin_amdgcn_global_load_lds((glb_ptr_t)(kb_ + ko_), (lds_ptr_t)(lk_ + u * 1024), 16, 0, 0);      \
-        __builtin_amdgcn_global_load_lds((glb_ptr_t)(vb_ + v_lane + u * 1024), (lds_ptr_t)(lv_ + u * 1024), 16, 0, 0); \
       }                                                                                                       \
+      _Pragma("unroll") for (int u = 0; u < WLV; u++)                                                         \
+        __builtin_amdgcn_global_load_lds((glb_ptr_t)(vb_ + v_lane + u * 1024), (lds_ptr_t)(lv_ + u * 1024), 16, 0, 0); \
     }                                                                                                         \
   }
 
@@ -181,6 +195,8 @@ __global__ __launch_bounds__(256, 3) void block_sparse_attn_kernel(const AttnPar
   const int vsw = v_swz(r);                // v_swz(32*dt + r) does not depend on dt
   // V^T operand: key chunks 2hh and 2hh+1 of channel row r (+32*dt); the two swizzled slots differ in bit 4 only
   const uint32_t v_rd_lo = (uint32_t)(r * 64 + (((2 * hh) ^ vsw) * 16));
+  // fp16 V^T operand of key step s: chunk (4hh + s) ^ (r & 7) of the 128-byte row r (+32*dt): v_rd16 ^ (16 * s)
+  const uint32_t v_rd16 = (uint32_t)(r * 128 + (((4 * hh) ^ (r & 7)) * 16));
 
   float m = SPG_NEG_BIG;
   float dsum = hh == 0 ? 1.0f : 0.0f;     // the two half-lanes of a query share d = 1.0 (sm89.cuh:172)
@@ -296,13 +312,57 @@ __global__ __launch_bounds__(256, 3) void block_sparse_attn_kernel(const AttnPar
     }
     if (compute) {
       cnt++;
-      const float neg = -m + SPG_FP8_OFFSET;
+      const float neg = PV16 ? -m : -m + SPG_FP8_OFFSET;
       float ps = 0.f;
 #pragma unroll
       for (int e = 0; e < 32; e++) {
         x[e] = __builtin_amdgcn_exp2f(__builtin_fmaf(x[e], a, neg));
-        ps += x[e];
+        if constexpr (!PV16) ps += x[e];
       }
+      if constexpr (PV16) {
+        typedef _Float16 h8 __attribute__((ext_vector_type(8)));
+        typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+        typedef float f2 __attribute__((ext_vector_type(2)));
+        h8 pb16[4];
+#pragma unroll
+        for (int s4 = 0; s4 < 4; s4++)
+#pragma unroll
+          for (int j = 0; j < 8; j += 2) {
+            const f2 pr = {x[8 * s4 + j], x[8 * s4 + j + 1]};
+            const h2 ph = __builtin_convertvector(pr, h2);          // v_cvt_pk_f16_f32, round to nearest even
+            pb16[s4][j] = ph[0];
+            pb16[s4][j + 1] = ph[1];
+            ps += (float)ph[0] + (float)ph[1];
+          }
+        dsum += ps;
+        const uint32_t va = lds_v0 + 2 * bufoff + v_rd16;
+        v4i t[4][NDT];
+        // steps 0,1 are read first; steps 2,3 are in flight while 0,1 multiply
+#pragma unroll
+        for (int s4 = 0; s4 < 2; s4++) {
+          lds_read_2x128<0, 4096>(t[s4][0], t[s4][1], va ^ (uint32_t)(16 * s4));
+          if constexpr (NDT == 4) lds_read_2x128<8192, 12288>(t[s4][2], t[s4][3], va ^ (uint32_t)(16 * s4));
+        }
+        if constexpr (NDT == 4) { lds_wait4(t[0][0], t[0][1], t[0][2], t[0][3]); lds_wait4(t[1][0], t[1][1], t[1][2], t[1][3]); }
+        else { lds_wait4(t[0][0], t[0][1], t[1][0], t[1][1]); }
+#pragma unroll
+        for (int s4 = 2; s4 < 4; s4++) {
+          lds_read_2x128<0, 4096>(t[s4][0], t[s4][1], va ^ (uint32_t)(16 * s4));
+          if constexpr (NDT == 4) lds_read_2x128<8192, 12288>(t[s4][2], t[s4][3], va ^ (uint32_t)(16 * s4));
+        }
+#pragma unroll
+        for (int s4 = 0; s4 < 2; s4++)
+#pragma unroll
+          for (int dt = 0; dt < NDT; dt++)
+            O[dt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(h8, t[s4][dt]), pb16[s4], O[dt], 0, 0, 0);
+        if constexpr (NDT == 4) { lds_wait4(t[2][0], t[2][1], t[2][2], t[2][3]); lds_wait4(t[3][0], t[3][1], t[3][2], t[3][3]); }
+        else { lds_wait4(t[2][0], t[2][1], t[3][0], t[3][1]); }
+#pragma unroll
+        for (int s4 = 2; s4 < 4; s4++)
+#pragma unroll
+          for (int dt = 0; dt < NDT; dt++)
+            O[dt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(h8, t[s4][dt]), pb16[s4], O[dt], 0, 0, 0);
+      } else {
       dsum += ps;
       v8i pb;
 #pragma unroll
@@ -343,6 +403,7 @@ __global__ __launch_bounds__(256, 3) void block_sparse_attn_kernel(const AttnPar
           O[dt] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(av, pb, O[dt], 0, 0, 0, 0, 0, 0);
         }
       }
+      }   // !PV16
     }
     // advance the block pipeline and the ring
     blk = blk1; blk1 = blk2; blk2 = blk2 + d3; d3 = d4;
@@ -365,7 +426,8 @@ __global__ __launch_bounds__(256, 3) void block_sparse_attn_kernel(const AttnPar
 #pragma unroll
       for (int g = 0; g < 4; g++) {
         const int d0 = 32 * dt + 8 * g + 4 * hh;
-        const float4 sc = *(const float4 *)(vs + d0);
+        float4 sc = make_float4(1.f, 1.f, 1.f, 1.f);
+        if constexpr (!PV16) sc = *(const float4 *)(vs + d0);
         const uint16_t o0 = f32_to_elem<ODT>(O[dt][4 * g + 0] * inv * sc.x);
         const uint16_t o1 = f32_to_elem<ODT>(O[dt][4 * g + 1] * inv * sc.y);
         const uint16_t o2 = f32_to_elem<ODT>(O[dt][4 * g + 2] * inv * sc.z);
@@ -389,12 +451,22 @@ hipError_t launch_block_sparse_attn(const int8_t *q8, const int8_t *k8, const ui
   p.total_wg = p.nq * H * B;
   p.wg_per_xcd = (p.total_wg + 7) / 8;
   const int grid = p.wg_per_xcd * 8;
-  if (D == 64) {
-    if (out_dtype == 0) block_sparse_attn_kernel<64, 0><<<grid, 256, 0, st>>>(p);
-    else block_sparse_attn_kernel<64, 1><<<grid, 256, 0, st>>>(p);
-  } else {
-    if (out_dtype == 0) block_sparse_attn_kernel<128, 0><<<grid, 256, 0, st>>>(p);
-    else block_sparse_attn_kernel<128, 1><<<grid, 256, 0, st>>>(p);
+  if (v_scale != nullptr) {
+    if (D == 64) {
+      if (out_dtype == 0) block_sparse_attn_kernel<64, 0, false><<<grid, 256, 0, st>>>(p);
+      else block_sparse_attn_kernel<64, 1, false><<<grid, 256, 0, st>>>(p);
+    } else {
+      if (out_dtype == 0) block_sparse_attn_kernel<128, 0, false><<<grid, 256, 0, st>>>(p);
+      else block_sparse_attn_kernel<128, 1, false><<<grid, 256, 0, st>>>(p);
+    }
+  } else {   // fp16 V^T tiles, no V scale
+    if (D == 64) {
+      if (out_dtype == 0) block_sparse_attn_kernel<64, 0, true><<<grid, 256, 0, st>>>(p);
+      else block_sparse_attn_kernel<64, 1, true><<<grid, 256, 0, st>>>(p);
+    } else {
+      if (out_dtype == 0) block_sparse_attn_kernel<128, 0, true><<<grid, 256, 0, st>>>(p);
+      else block_sparse_attn_kernel<128, 1, true><<<grid, 256, 0, st>>>(p);
+    }
   }
   return hipGetLastError();
 }

@@ -134,6 +134,29 @@ int spg_block_sparse_attn(const int8_t *q8, const int8_t *k8, const uint8_t *v8,
                                                         is_causal ? 1 : 0, pv_count, (hipStream_t)stream));
 }
 
+int spg_v_tiles_f16(const void *v, void *vt, int B, int H, int N, int D, int dtype, void *stream) {
+  const char *fn = "spg_v_tiles_f16";
+  SPG_TRY(check_shape(fn, B, H, N, D));
+  SPG_TRY(check_dtype(fn, dtype));
+  SPG_NONNULL(fn, v); SPG_NONNULL(fn, vt);
+  spg::launch_v_tiles_f16(v, vt, B, H, N, D, dtype, (hipStream_t)stream);
+  return check_launch(fn, hipSuccess);
+}
+
+int spg_block_sparse_attn_f16v(const int8_t *q8, const int8_t *k8, const void *vt, void *out, int out_dtype,
+                               const int32_t *lut, const int32_t *valid_block_num, const float *pvthreshd,
+                               const float *q_scale, const float *k_scale, int B, int H, int N, int D, float sm_scale,
+                               int is_causal, int32_t *pv_count, void *stream) {
+  const char *fn = "spg_block_sparse_attn_f16v";
+  SPG_TRY(check_shape(fn, B, H, N, D));
+  SPG_TRY(check_dtype(fn, out_dtype));
+  SPG_NONNULL(fn, q8); SPG_NONNULL(fn, k8); SPG_NONNULL(fn, vt); SPG_NONNULL(fn, out); SPG_NONNULL(fn, lut);
+  SPG_NONNULL(fn, valid_block_num); SPG_NONNULL(fn, pvthreshd); SPG_NONNULL(fn, q_scale); SPG_NONNULL(fn, k_scale);
+  return check_launch(fn, spg::launch_block_sparse_attn(q8, k8, (const uint8_t *)vt, out, out_dtype, lut, valid_block_num,
+                                                        pvthreshd, q_scale, k_scale, nullptr, B, H, N, D, sm_scale,
+                                                        is_causal ? 1 : 0, pv_count, (hipStream_t)stream));
+}
+
 int spg_dense_attn_f16(const void *q, const void *k, const void *v, void *out, int B, int H, int N, int D,
                        float sm_scale, int is_causal, void *stream) {
   const char *fn = "spg_dense_attn_f16";

@@ -21,6 +21,8 @@ hipError_t launch_map_to_lut(const void *mask, int kind, int32_t *lut, int32_t *
 void launch_v_quant_fp8(const void *v, uint8_t *v8, float *v_scale, int B, int H, int N, int D, int dtype,
                         hipStream_t st);
 
+void launch_v_tiles_f16(const void *v, void *vt, int B, int H, int N, int D, int dtype, hipStream_t st);
+
 hipError_t launch_block_sparse_attn(const int8_t *q8, const int8_t *k8, const uint8_t *v8, void *out, int out_dtype,
                                     const int32_t *lut, const int32_t *valid, const float *pvthreshd,
                                     const float *q_scale, const float *k_scale, const float *v_scale, int B, int H,

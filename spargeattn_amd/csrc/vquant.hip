@@ -99,6 +99,47 @@ __global__ __launch_bounds__(256) void v_quant_kernel(const uint16_t *__restrict
   }
 }
 
+// V -> fp16 -> V^T tiles [nk][D][64] fp16 for the fp16-PV attention variant.  Inside a 128-byte tile row (one channel,
+// 64 keys) the eight 8-key chunks are stored at slot = chunk ^ (d & 7) (the LDS swizzle of the attention kernel).
+// Keys at or beyond N are zero.  One workgroup per 64-key tile.
+template <int D, int DT>
+__global__ __launch_bounds__(256) void v_tiles_f16_kernel(const uint16_t *__restrict__ v, uint16_t *__restrict__ vt,
+                                                          int N, int nk) {
+  constexpr int TPR = D / 8;
+  constexpr int RPP = 256 / TPR;
+  constexpr int NP = 64 / RPP;
+  constexpr int LDW = 64 + 2;  // padded row (halves) of the transposed tile
+  __shared__ __align__(16) uint16_t tile[D * LDW];
+  const int blk = blockIdx.x, bh = blockIdx.y, tid = threadIdx.x;
+  const int c = tid % TPR, r = tid / TPR;
+  const uint16_t *base = v + ((size_t)bh * N + (size_t)blk * 64) * D + c * 8;
+#pragma unroll
+  for (int p = 0; p < NP; p++) {
+    const int row = r + p * RPP;
+    uint4 q = make_uint4(0, 0, 0, 0);
+    if (blk * 64 + row < N) q = *(const uint4 *)(base + (size_t)row * D);
+    const uint32_t w[4] = {q.x, q.y, q.z, q.w};
+#pragma unroll
+    for (int e = 0; e < 8; e++) {
+      const uint16_t b = (uint16_t)((e & 1) ? (w[e >> 1] >> 16) : (w[e >> 1] & 0xffffu));
+      uint16_t h = b;
+      if constexpr (DT == 1) h = f32_to_elem<0>(elem_to_f32<1>(b));     // bf16 -> fp16, one rounding
+      tile[(c * 8 + e) * LDW + row] = h;
+    }
+  }
+  __syncthreads();
+  uint16_t *out = vt + ((size_t)bh * nk + blk) * (size_t)(D * 64);
+  for (int i = tid; i < D * 8; i += 256) {   // 16-byte pieces: D rows x 8 slots
+    const int d = i >> 3, slot = i & 7;
+    const int kc = slot ^ (d & 7);             // key chunk stored in this slot
+    const uint16_t *src = tile + d * LDW + kc * 8;
+    uint32_t o[4];
+#pragma unroll
+    for (int e = 0; e < 4; e++) o[e] = (uint32_t)src[2 * e] | ((uint32_t)src[2 * e + 1] << 16);
+    *(uint4 *)(out + d * 64 + slot * 8) = make_uint4(o[0], o[1], o[2], o[3]);
+  }
+}
+
 __global__ void v_scale_final_kernel(float *v_scale, int n) {
   const int i = blockIdx.x * blockDim.x + threadIdx.x;
   if (i < n) v_scale[i] = v_scale[i] / 2.25f;
@@ -127,6 +168,15 @@ void launch_v_quant_fp8(const void *v, uint8_t *v8, float *v_scale, int B, int H
                         hipStream_t st) {
   if (D == 64) { if (dtype == 0) launch_vq2<64, 0>(v, v8, v_scale, B, H, N, st); else launch_vq2<64, 1>(v, v8, v_scale, B, H, N, st); }
   else         { if (dtype == 0) launch_vq2<128, 0>(v, v8, v_scale, B, H, N, st); else launch_vq2<128, 1>(v, v8, v_scale, B, H, N, st); }
+}
+
+void launch_v_tiles_f16(const void *v, void *vt, int B, int H, int N, int D, int dtype, hipStream_t st) {
+  const int nk = (N + 63) / 64;
+  const dim3 grid(nk, B * H);
+  const uint16_t *vp = (const uint16_t *)v;
+  uint16_t *op = (uint16_t *)vt;
+  if (D == 64) { if (dtype == 0) v_tiles_f16_kernel<64, 0><<<grid, 256, 0, st>>>(vp, op, N, nk); else v_tiles_f16_kernel<64, 1><<<grid, 256, 0, st>>>(vp, op, N, nk); }
+  else         { if (dtype == 0) v_tiles_f16_kernel<128, 0><<<grid, 256, 0, st>>>(vp, op, N, nk); else v_tiles_f16_kernel<128, 1><<<grid, 256, 0, st>>>(vp, op, N, nk); }
 }
 
 }  // namespace spg

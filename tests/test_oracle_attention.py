@@ -123,3 +123,61 @@ def test_topk_api_end_to_end_small():
     assert list(res_c["valid"][0, 0]) == [2, 4, 6, 8, 8, 8, 8, 8]
     tot = float(res_c["valid"].sum())
     assert abs(res_c["sparsity"] - (1 - tot / (9 * 8 * 2))) < 1e-12      # causal denominator (nk+2)//2
+
+
+# ---- SageAttention1 variant (INT8 QK^T, FP16 PV): pinned by the same library-routine special cases ----------------
+
+def _dequantised_f16v(res, n):
+    q = res["q8"].astype(np.float64) * np.repeat(res["q_scale"].astype(np.float64), 128, axis=2)[:, :, :n, None]
+    k = res["k8"].astype(np.float64) * np.repeat(res["k_scale"].astype(np.float64), 64, axis=2)[:, :, :n, None]
+    return torch.from_numpy(q), torch.from_numpy(k), torch.from_numpy(res["v16"][:, :, :n].astype(np.float64))
+
+
+@pytest.mark.parametrize("tag,d,n", [(R.BF16, 128, 384), (R.FP16, 64, 300)])
+def test_f16v_all_blocks_reduces_to_dense_sdpa(tag, d, n):
+    q, k, v = _inputs(10, 1, 2, n, d, tag)
+    res = api.spas_sage_attn_meansim_topk(q, k, v, tag, topk=1.0)
+    assert res["map"].all() and np.array_equal(res["pv_count"], res["valid"])
+    assert np.array_equal(res["v16"][:, :, :n], v.astype(np.float16).astype(np.float32))
+    qd, kd, vd = _dequantised_f16v(res, n)
+    ref = torch.nn.functional.scaled_dot_product_attention(qd, kd, vd).numpy()
+    met = at.precision_metric(res["out"], ref)
+    # remaining error: fp16 rounding of P (numerator and denominator alike) and the output rounding: far below the
+    # e4m3 variant's
+    assert met["Cossim"] > 0.99999 and met["L1"] < (6e-3 if tag == R.BF16 else 1.5e-3), met
+
+
+def test_f16v_token_causal_and_block_mask():
+    tag, d, n = R.FP16, 64, 512
+    q, k, v = _inputs(11, 1, 2, n, d, tag)
+    res = api.spas_sage_attn_meansim_topk(q, k, v, tag, topk=0.5, is_causal=True)
+    qd, kd, vd = _dequantised_f16v(res, n)
+    tok = _token_mask(res["map"], n) & torch.tril(torch.ones(n, n, dtype=torch.bool))
+    ref = torch.nn.functional.scaled_dot_product_attention(qd, kd, vd, attn_mask=tok).numpy()
+    met = at.precision_metric(res["out"], ref)
+    assert met["Cossim"] > 0.99999 and met["L1"] < 1.5e-3, met
+    # sparsity is reported against the causal denominator (core.py:314-317)
+    assert abs(res["sparsity"] - (1 - res["valid"].sum() / ((8 + 2) // 2 * 4 * 2))) < 1e-12
+
+
+def test_f16v_denominator_uses_rounded_p():
+    """One dominant key (p = 1, v = 1) and 63 999 keys whose probability 1.4 * 2^-24 rounds to the fp16 subnormal 2^-24
+    (v = 0): the output is 1 / (1 + 63999 * 2^-24) = 0.99620 when the denominator sums the ROUNDED P and 0.99469 when
+    it sums the exact P; fp16 resolves the two."""
+    d, nblk = 64, 1000
+    n = 64 * nblk
+    q8 = np.zeros((1, 1, 128, d), np.int8); q8[0, 0, :, 0] = 100
+    k8 = np.zeros((1, 1, n, d), np.int8); k8[0, 0, 0, 0] = 100
+    v16 = np.zeros((1, 1, n, d), np.float32); v16[0, 0, 0, :] = 1.0
+    lut = np.ones((1, 1, 1, nblk), np.int32); lut[0, 0, 0, 0] = 0
+    valid = np.full((1, 1, 1), nblk, np.int32)
+    target = 1.4 * 2.0 ** -24
+    c = -np.log(target) / 10000.0                         # softmax scale: exp(-10000 c) = target
+    out, written, pvc = at.block_sparse_attention(
+        q8, k8, v16, lut, valid, np.array([50.0], np.float32), np.full((1, 1, 1), 0.1, np.float32),
+        np.full((1, 1, nblk), 0.1, np.float32), None, c / 0.01, "fp16", return_pv_count=True, pv="f16")
+    assert pvc[0, 0, 0] == nblk
+    rounded = 1.0 / (1.0 + (n - 1) * 2.0 ** -24)
+    exact = 1.0 / (1.0 + (n - 1) * target)
+    got = float(out[0, 0, 5, 3])
+    assert abs(got - rounded) < 4e-4 < abs(got - exact), (got, rounded, exact)
