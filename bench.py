@@ -22,6 +22,7 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 PEAK_MFMA_8BIT = 5.0e15   # MI355X dense INT8 = FP8 MFMA peak, op/s
+PEAK_MFMA_F16 = 2.5e15    # MI355X dense FP16 MFMA peak, flop/s
 PEAK_HBM = 8.0e12
 # HBM-side bytes per launch of the attention kernel, measured with two rocprofv3 --pmc runs (FETCH_SIZE, WRITE_SIZE,
 # each scaled by what the same counter reads for a 1 GiB device copy: x2.0 and x1.0).  Only known for the workload
@@ -35,6 +36,8 @@ def parse():
     ap.add_argument("--steps", type=int, default=10)
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--config", default="cfg4", help="workload (cfg1..cfg5); the headline is cfg4")
+    ap.add_argument("--api", default="sage2", choices=["sage2", "sage1"],
+                    help="sage2: INT8 QK^T + FP8 PV (headline); sage1: INT8 QK^T + FP16 PV (spas_sage_attn_meansim_topk_cuda)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-dense", action="store_true")
     ap.add_argument("--copy-calibration", action="store_true",
@@ -95,9 +98,13 @@ def main():
     nq, nk = (N + 127) // 128, (N + 63) // 64
     dense_flop = 4.0 * B * H * N * N * D * (0.5 if cfg.is_causal else 1.0)
 
+    sage1 = args.api == "sage1"
+    op = sa.spas_sage_attn_meansim_topk_cuda if sage1 else sa.spas_sage2_attn_meansim_topk_cuda
+    # executed ops split evenly between the two products: the blended MFMA peak is the harmonic mean of their peaks
+    peak_mfma = 2.0 / (1.0 / PEAK_MFMA_8BIT + 1.0 / PEAK_MFMA_F16) if sage1 else PEAK_MFMA_8BIT
+
     def step():
-        return sa.spas_sage2_attn_meansim_topk_cuda(q, k, v, is_causal=cfg.is_causal, topk=cfg.topk,
-                                                    pvthreshd=cfg.pvthreshd)
+        return op(q, k, v, is_causal=cfg.is_causal, topk=cfg.topk, pvthreshd=cfg.pvthreshd)
 
     # ---- stage events (recorded on the stream the kernels are launched on) -------------------------------
     names = ["km", "maskpred", "vquant", "attn", "end"]
@@ -118,10 +125,15 @@ def main():
         from spargeattn_amd import utils
         lut, valid, q8, qs, k8, ks = utils.get_block_map_meansim_fuse_quant(
             q, k, km, is_causal=cfg.is_causal, simthreshd1=-0.1, cdfthreshd=None, topk=cfg.topk, return_lut=True)
-        v8, vs = _lib.v_quant_fp8(v.to(torch.float16))
         o = torch.empty_like(q)
         pvt = torch.full((H,), float(cfg.pvthreshd), device=dev)
-        run = lambda: _lib.block_sparse_attn(q8, k8, v8, o, lut, valid, pvt, qs, ks, vs, 1.0 / D ** 0.5)
+        if sage1:
+            vt = _lib.v_tiles_f16_swizzled(v)
+            run = lambda: _lib.block_sparse_attn_f16v(q8, k8, vt, o, lut, valid, pvt, qs, ks, 1.0 / D ** 0.5,
+                                                      is_causal=cfg.is_causal)
+        else:
+            v8, vs = _lib.v_quant_fp8(v.to(torch.float16))
+            run = lambda: _lib.block_sparse_attn(q8, k8, v8, o, lut, valid, pvt, qs, ks, vs, 1.0 / D ** 0.5)
         for _ in range(args.warmup):
             run()
         torch.cuda.synchronize()
@@ -174,23 +186,26 @@ def main():
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": step_s * 1e3,
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": "int8 QK^T + fp8-e4m3 PV (fp32 softmax/accumulate), bf16 in/out",
+        "dtype": ("int8 QK^T + fp16 PV" if sage1 else "int8 QK^T + fp8-e4m3 PV") + " (fp32 softmax/accumulate), bf16 in/out",
         "data": "synthetic (seeded generator, see spargeattn_amd/workloads.py)",
-        "config": {"workload": f"{cfg.name}: spas_sage2_attn_meansim_topk_cuda B={B} H={H} N={N} D={D} "
+        "config": {"workload": f"{cfg.name}: {op.__name__} B={B} H={H} N={N} D={D} "
                                f"{'causal' if cfg.is_causal else 'non-causal'} topk={cfg.topk} pvthreshd={cfg.pvthreshd}",
                    "selected_blocks": sel_blocks, "block_density": sel_blocks / (B * H * nq * nk)},
         "attn_kernel": {"ms": stage_ms["attn"], "dense_equiv_tops": dense_flop / attn_s / 1e12,
                         "executed_tops": executed_ops / attn_s / 1e12,
-                        "mfma_util_pct": 100.0 * executed_ops / attn_s / PEAK_MFMA_8BIT},
+                        "mfma_util_pct": 100.0 * executed_ops / attn_s / peak_mfma},
         "mask_pred": {"us": mp_ms * 1e3, "km_us": stage_ms["km"] * 1e3, "pool_quant_select_us": stage_ms["maskpred"] * 1e3,
                       "algorithmic_GB": mp_bytes / 1e9, "GBps": mp_bytes / (mp_ms * 1e-3) / 1e9,
                       "hbm_frac": mp_bytes / (mp_ms * 1e-3) / PEAK_HBM},
         "v_quant": {"us": stage_ms["vquant"] * 1e3, "GBps": vq_bytes / (stage_ms["vquant"] * 1e-3) / 1e9},
-        "roofline": {"kernel": "block_sparse_attn_kernel<128,bf16>", "bound": "mfma",
-                     "achieved": executed_ops / attn_s / 1e12, "peak": PEAK_MFMA_8BIT / 1e12, "unit": "TFLOP/s",
-                     "frac": executed_ops / attn_s / PEAK_MFMA_8BIT, "traffic": MEASURED_ATTN_TRAFFIC.get(cfg.name),
-                     "note": "achieved = executed INT8+FP8 MFMA ops (selected blocks * 2*128*64*D*2) / HIP-event time of "
-                             "the kernel inside the timed steps; peak = MI355X dense 8-bit MFMA"},
+        "roofline": {"kernel": f"block_sparse_attn_kernel<{D},{'bf16' if q.dtype == torch.bfloat16 else 'fp16'},{'fp16 PV' if sage1 else 'fp8 PV'}>",
+                     "bound": "mfma",
+                     "achieved": executed_ops / attn_s / 1e12, "peak": peak_mfma / 1e12, "unit": "TFLOP/s",
+                     "frac": executed_ops / attn_s / peak_mfma,
+                     "traffic": None if sage1 else MEASURED_ATTN_TRAFFIC.get(cfg.name),
+                     "note": "achieved = executed MFMA ops of both products (selected blocks * 2*128*64*D*2) / HIP-event time "
+                             "of the kernel inside the timed steps; peak = MI355X dense 8-bit MFMA"
+                             + (" for QK^T and dense fp16 MFMA for PV, blended" if sage1 else "")},
     }
 
     if not args.no_dense:
