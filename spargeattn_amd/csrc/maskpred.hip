@@ -175,6 +175,11 @@ __global__ __launch_bounds__(256) void pool_sim_quant_kernel(const uint16_t *__r
     double colsum[8], colxh[8];
 #pragma unroll
     for (int e = 0; e < 8; e++) { colsum[e] = 0.0; colxh[e] = 0.0; }
+    // row norms: the TPR lanes of a row group all need sqrt(sum of squares) and its reciprocal for each of their NP
+    // rows.  Both are computed ONCE per NP rows - lane c of the group takes row c % NP - and handed round with lane
+    // reads, instead of NP times in every lane.
+    static_assert(NP <= TPR, "one lane of the row group per row");
+    float ssf_mine = 0.f;
 #pragma unroll
     for (int p = 0; p < NP; p++) {
       double ss = 0.0;
@@ -185,9 +190,17 @@ __global__ __launch_bounds__(256) void pool_sim_quant_kernel(const uint16_t *__r
         colsum[e] += xd;
       }
       ss = group_sum_f64<TPR>(ss);                 // the TPR lanes of this row
-      const float norm = sqrtf((float)ss);
+      const float ssf = (float)ss;
+      ssf_mine = (c % NP == p) ? ssf : ssf_mine;
+    }
+    const float norm_mine = sqrtf(ssf_mine);
+    const float rn_mine = rcp_safe(norm_mine) ? exact_rcp(norm_mine) : 0.f;
+    const int group_lane0 = (tid & 63) & ~(TPR - 1);
+#pragma unroll
+    for (int p = 0; p < NP; p++) {
+      const float norm = __shfl(norm_mine, group_lane0 + p, SPG_WAVE);
+      const float rn = __shfl(rn_mine, group_lane0 + p, SPG_WAVE);
       if (rcp_safe(norm)) {
-        const float rn = exact_rcp(norm);
 #pragma unroll
         for (int e = 0; e < 8; e++) {
           const _Float16 h = (_Float16)div_by(xf[p][e], norm, rn);
