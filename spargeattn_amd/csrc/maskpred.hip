@@ -135,14 +135,18 @@ __global__ __launch_bounds__(256) void pool_sim_quant_kernel(const uint16_t *__r
     }
   }
 
+  // all loads of the thread are issued before the first use (rows beyond the block's end re-read its last row and
+  // are zeroed afterwards: no load sits behind a branch)
+  uint4 raw[NP];
+#pragma unroll
+  for (int p = 0; p < NP; p++) raw[p] = *(const uint4 *)(xb + (size_t)min(r + p * RPP, rows_valid - 1) * D);
   float xf[NP][8];
   float amax = 0.f;
 #pragma unroll
   for (int p = 0; p < NP; p++) {
     const int row = r + p * RPP;
     const bool ok = row < rows_valid;
-    uint4 v = make_uint4(0, 0, 0, 0);
-    if (ok) v = *(const uint4 *)(xb + (size_t)row * D);
+    const uint4 v = ok ? raw[p] : make_uint4(0, 0, 0, 0);
     const uint32_t w[4] = {v.x, v.y, v.z, v.w};
 #pragma unroll
     for (int e = 0; e < 8; e += 2) {
