@@ -73,12 +73,15 @@ __global__ __launch_bounds__(256) void v_quant_kernel(const uint16_t *__restrict
 #pragma unroll
   for (int e = 0; e < 8; e++) recp[e] = 2.25f / amax[(size_t)bh * D + c * 8 + e];
   const uint16_t *base = v + ((size_t)bh * N + (size_t)blk * 64) * D + c * 8;
+  const int last_row = min(63, N - 1 - blk * 64);
+  uint4 raw[NP];                     // every load is issued before the first use; rows beyond N re-read the last row
+#pragma unroll
+  for (int p = 0; p < NP; p++) raw[p] = *(const uint4 *)(base + (size_t)min(r + p * RPP, last_row) * D);
 #pragma unroll
   for (int p = 0; p < NP; p++) {
     const int row = r + p * RPP;
-    const bool ok = blk * 64 + row < N;
-    uint4 q = make_uint4(0, 0, 0, 0);
-    if (ok) q = *(const uint4 *)(base + (size_t)row * D);
+    const bool ok = row <= last_row;
+    const uint4 q = raw[p];
     const uint32_t w[4] = {q.x, q.y, q.z, q.w};
 #pragma unroll
     for (int e = 0; e < 8; e += 2) {
@@ -113,11 +116,14 @@ __global__ __launch_bounds__(256) void v_tiles_f16_kernel(const uint16_t *__rest
   const int blk = blockIdx.x, bh = blockIdx.y, tid = threadIdx.x;
   const int c = tid % TPR, r = tid / TPR;
   const uint16_t *base = v + ((size_t)bh * N + (size_t)blk * 64) * D + c * 8;
+  const int last_row = min(63, N - 1 - blk * 64);
+  uint4 raw[NP];
+#pragma unroll
+  for (int p = 0; p < NP; p++) raw[p] = *(const uint4 *)(base + (size_t)min(r + p * RPP, last_row) * D);
 #pragma unroll
   for (int p = 0; p < NP; p++) {
     const int row = r + p * RPP;
-    uint4 q = make_uint4(0, 0, 0, 0);
-    if (blk * 64 + row < N) q = *(const uint4 *)(base + (size_t)row * D);
+    const uint4 q = row <= last_row ? raw[p] : make_uint4(0, 0, 0, 0);
     const uint32_t w[4] = {q.x, q.y, q.z, q.w};
 #pragma unroll
     for (int e = 0; e < 8; e++) {
