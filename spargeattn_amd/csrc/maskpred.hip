@@ -700,14 +700,40 @@ __global__ __launch_bounds__(256) void block_select_wave_kernel(
       okey[t] = j < nk ? ((bits << 16) | (0xffffu - (uint32_t)j)) : 0u;
       key[t] = okey[t];
     }
-    bitonic_sort_desc<EPL, 2>(key, lane);             // sorted position of key[t] is lane * EPL + t
-
-    // how many to keep
+    // how many to keep, and the key of the last one kept
     long long n;
+    uint32_t kth = 0u;
     if (topk != nullptr) {
       const float t = topk[h] * (float)nk;            // binary32 product, truncated (utils.py:405)
       n = (long long)t;
+      if (n <= 0) n = 1;                              // utils.py:289
+      if (n < nk) {
+        // top-k needs the n-th largest key only, not the order: build it bit by bit, the largest T with
+        // #{key >= T} >= n.  Keys are distinct, probabilities are <= 1 (bits 31 and 30 of a key are clear) and
+        // bits 15 .. log2(NKP) are set in every real key (they hold 0xFFFF - column).
+        constexpr int LOW = 31 - __builtin_clz((unsigned)NKP);   // log2(NKP)
+        uint32_t T = 0u;
+        auto at_least_n = [&](uint32_t cand) {
+          int cnt = 0;
+#pragma unroll
+          for (int tt = 0; tt < EPL; tt++) cnt += __builtin_popcountll(__ballot(okey[tt] >= cand));
+          return cnt >= (int)n;
+        };
+#pragma unroll
+        for (int bit = 29; bit >= 16; bit--) {
+          const uint32_t cand = T | (1u << bit);
+          if (at_least_n(cand)) T = cand;
+        }
+        T |= 0xffffu & ~((1u << LOW) - 1u);
+#pragma unroll
+        for (int bit = LOW - 1; bit >= 0; bit--) {
+          const uint32_t cand = T | (1u << bit);
+          if (at_least_n(cand)) T = cand;
+        }
+        kth = T;
+      }
     } else {
+      bitonic_sort_desc<EPL, 2>(key, lane);           // sorted position of key[t] is lane * EPL + t
       // cdf[v] = T(sum_{u<=v} p_sorted[u]);  n = #{v < nk : cdf[v] <= threshold}  (utils.py:398-403)
       double lsum = 0.0;
 #pragma unroll
@@ -727,15 +753,14 @@ __global__ __launch_bounds__(256) void block_select_wave_kernel(
       }
       n = wave_sum_i32(cnt);
       __builtin_amdgcn_wave_barrier();
-    }
-    if (n <= 0) n = 1;                                // utils.py:289
-    uint32_t kth = 0u;
-    if (n < nk) {                                     // wavefront-uniform
-      const int pos = (int)n - 1, src = pos / EPL, tt = pos % EPL;
-      uint32_t mine = key[0];
+      if (n <= 0) n = 1;                              // utils.py:289
+      if (n < nk) {                                   // wavefront-uniform
+        const int pos = (int)n - 1, src = pos / EPL, tt = pos % EPL;
+        uint32_t mine = key[0];
 #pragma unroll
-      for (int t = 1; t < EPL; t++) mine = (tt == t) ? key[t] : mine;
-      kth = (uint32_t)__shfl((int)mine, src, SPG_WAVE);
+        for (int t = 1; t < EPL; t++) mine = (tt == t) ? key[t] : mine;
+        kth = (uint32_t)__shfl((int)mine, src, SPG_WAVE);
+      }
     }
 
     // block map row, ascending index list, delta LUT
