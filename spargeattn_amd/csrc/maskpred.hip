@@ -581,7 +581,11 @@ __global__ __launch_bounds__(256) void block_select_wave_kernel(
   int32_t *s_idx_all = (int32_t *)(smem + (size_t)R * D * 8 + (size_t)R * NKP * 4);   // [4][NKP]
   double *s_lsum_all = (double *)(smem + (size_t)R * D * 8 + (size_t)R * NKP * 4 + 4 * (size_t)NKP * 4);   // [4][64]
 
-  const int i0 = blockIdx.x * R, bh = blockIdx.y, h = bh % H, tid = threadIdx.x;
+  // Causal rows get heavier with the row index.  Workgroups that differ by 8 in blockIdx.y tend to share a CU (ids are
+  // dealt round-robin over 8 XCDs, then over the CUs of an XCD), so the row-group index is rotated by a quarter of
+  // the grid per such step: a CU then holds a mix of light and heavy row groups.
+  const int bx = (int)((blockIdx.x + (blockIdx.y >> 3) * (gridDim.x >> 2)) % gridDim.x);
+  const int i0 = bx * R, bh = blockIdx.y, h = bh % H, tid = threadIdx.x;
   const int rows = min(R, nq - i0);
   for (int t = tid; t < R * D; t += 256) {
     const int row = t / D;
@@ -606,17 +610,20 @@ __global__ __launch_bounds__(256) void block_select_wave_kernel(
       const uint4 *krow_a = (const uint4 *)(pk_base + (size_t)(live_a ? ja : 0) * D);
       const uint4 *krow_c = (const uint4 *)(pk_base + (size_t)(live_c ? jc : 0) * D);
       const bool two = jb + 256 < j_live;                            // workgroup-uniform
+      uint4 va_next = krow_a[0], vc_next = krow_c[0];
 #pragma unroll 1
       for (int cch = 0; cch < D / 8; cch++) {
-        const uint4 va = krow_a[cch];
+        const uint4 va = va_next, vc_cur = vc_next;
+        const int nxt = min(cch + 1, D / 8 - 1);                     // the next chunk is in flight during this one
+        va_next = krow_a[nxt];
+        vc_next = krow_c[nxt];
         const uint32_t wa[4] = {va.x, va.y, va.z, va.w};
         double ka[8];
 #pragma unroll
         for (int e = 0; e < 8; e++)
           ka[e] = (double)elem_to_f32<DT>((uint16_t)((e & 1) ? (wa[e >> 1] >> 16) : (wa[e >> 1] & 0xffffu)));
         if (two) {
-          const uint4 vc = krow_c[cch];
-          const uint32_t wc[4] = {vc.x, vc.y, vc.z, vc.w};
+          const uint32_t wc[4] = {vc_cur.x, vc_cur.y, vc_cur.z, vc_cur.w};
           double kc[8];
 #pragma unroll
           for (int e = 0; e < 8; e++)
