@@ -187,3 +187,32 @@ def test_dense_f16_comparator(D, N, causal):
     ref = torch.nn.functional.scaled_dot_product_attention(q.float(), k.float(), v.float(), is_causal=causal)
     met = oat.precision_metric(to_np(o), to_np(ref))
     assert met["Cossim"] > 0.9999 and met["L1"] < 5e-3, met
+
+
+def test_operator_under_hip_graph_capture():
+    """The C ABI neither allocates nor synchronises, so the operator can be captured; every replay (with eager work
+    and synchronisations in between) must reproduce the eager output bit for bit."""
+    cfg = W.CONFIGS["cfg1"]
+    q, k, v = W.make_qkv(cfg, device="cuda")
+    eager = sa.spas_sage2_attn_meansim_topk_cuda(q, k, v, topk=cfg.topk)
+    qs, ks, vs = q.clone(), k.clone(), v.clone()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):                       # warm-up on the capture stream
+        sa.spas_sage2_attn_meansim_topk_cuda(qs, ks, vs, topk=cfg.topk)
+    torch.cuda.current_stream().wait_stream(side)
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g):
+        out = sa.spas_sage2_attn_meansim_topk_cuda(qs, ks, vs, topk=cfg.topk)
+    for rep in range(3):
+        g.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out, eager), rep
+        other = sa.spas_sage2_attn_meansim_topk_cuda(q.flip(2).contiguous(), k, v, topk=cfg.topk)   # eager work between replays
+        torch.cuda.synchronize()
+        assert other.shape == eager.shape
+    # new inputs through the static buffers
+    qs.copy_(q.flip(2))
+    g.replay()
+    torch.cuda.synchronize()
+    assert torch.equal(out, sa.spas_sage2_attn_meansim_topk_cuda(q.flip(2).contiguous(), k, v, topk=cfg.topk))
