@@ -199,7 +199,9 @@ __global__ __launch_bounds__(256, PV16 ? 2 : 3) void block_sparse_attn_kernel(co
   const uint32_t v_rd16 = (uint32_t)(r * 128 + (((4 * hh) ^ (r & 7)) * 16));
 
   float m = SPG_NEG_BIG;
-  float dsum = hh == 0 ? 1.0f : 0.0f;     // the two half-lanes of a query share d = 1.0 (sm89.cuh:172)
+  // d = 1.0 initially (sm89.cuh:172).  FP8 path: each half-lane sums its own 32 keys, so only one of the two starts at 1;
+  // FP16 path: both half-lanes hold the full row sum.
+  float dsum = (PV16 || hh == 0) ? 1.0f : 0.0f;
   v16f O[NDT];
 #pragma unroll
   for (int dt = 0; dt < NDT; dt++)
@@ -332,9 +334,18 @@ __global__ __launch_bounds__(256, PV16 ? 2 : 3) void block_sparse_attn_kernel(co
             const h2 ph = __builtin_convertvector(pr, h2);          // v_cvt_pk_f16_f32, round to nearest even
             pb16[s4][j] = ph[0];
             pb16[s4][j + 1] = ph[1];
-            ps += (float)ph[0] + (float)ph[1];
           }
-        dsum += ps;
+        {
+          // row sums of the ROUNDED P on the matrix unit, as the reference does (rowsum_f16f16f32, attn_utils.cuh:614):
+          // ones (32 x 16) . P^T gives, in every row, the sum over the 16 keys of the step for each query column
+          const h8 ones = {(_Float16)1, (_Float16)1, (_Float16)1, (_Float16)1, (_Float16)1, (_Float16)1, (_Float16)1, (_Float16)1};
+          v16f dacc;
+#pragma unroll
+          for (int e = 0; e < 16; e++) dacc[e] = 0.f;
+#pragma unroll
+          for (int s4 = 0; s4 < 4; s4++) dacc = __builtin_amdgcn_mfma_f32_32x32x16_f16(ones, pb16[s4], dacc, 0, 0, 0);
+          dsum += dacc[0];                 // all 64 keys of the block, identical in both half-lanes of the query
+        }
         const uint32_t va = lds_v0 + 2 * bufoff + v_rd16;
         v4i t[4][NDT];
         // steps 0,1 are read first; steps 2,3 are in flight while 0,1 multiply
@@ -416,7 +427,7 @@ __global__ __launch_bounds__(256, PV16 ? 2 : 3) void block_sparse_attn_kernel(co
   if (p.pv_count != nullptr && tid == 0) p.pv_count[(size_t)bh * p.nq + qb] = cnt;
 
   // ---- epilogue: O / d * v_scale -> out dtype -----------------------------------------------------------
-  const float dtot = half_swap_sum_f32(dsum);
+  const float dtot = PV16 ? dsum : half_swap_sum_f32(dsum);
   const float inv = __builtin_amdgcn_rcpf(dtot);
   if (q_row < N) {
     uint16_t *orow = (uint16_t *)p.out + ((size_t)bh * N + q_row) * D;
