@@ -90,7 +90,9 @@ int spg_v_quant_fp8(const void *v, uint8_t *v8, float *v_scale, int B, int H, in
  * tensor_layout = HND, qk_quant_gran = per-block, PV threshold per block.
  * q8,k8 int8 (B,H,N,D); v8 as produced by spg_v_quant_fp8; out (B,H,N,D) out_dtype;
  * lut/valid_block_num as above; pvthreshd (H,) float32; q_scale (B,H,nq), k_scale (B,H,nk),
- * v_scale (B,H,D) float32; pv_count (B,H,nq) int32 or NULL (number of K blocks whose PV was computed).
+ * v_scale (B,H,D) float32; pv_count (B,H,nq*4) int32 or NULL: number of K blocks
+ * whose PV was computed, one entry per 32 query rows as in the reference (sm89.cu:331-334); entries of Q blocks with
+ * valid_block_num == 0 are left untouched.
  * Row blocks with valid_block_num == 0 are left unwritten, as in the reference (sm89.cuh:232-235). */
 int spg_block_sparse_attn(const int8_t *q8, const int8_t *k8, const uint8_t *v8, void *out, int out_dtype,
                           const int32_t *lut, const int32_t *valid_block_num, const float *pvthreshd,

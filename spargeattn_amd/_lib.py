@@ -196,7 +196,7 @@ def block_sparse_attn(q8, k8, v8, out, lut, valid, pvthreshd, q_scale, k_scale, 
                       is_causal=False, return_pv_count=False):
     _dev(q8, k8, v8, out, lut, valid, pvthreshd, q_scale, k_scale, v_scale)
     B, H, N, D = q8.shape
-    pvc = torch.zeros((B, H, (N + 127) // 128), dtype=torch.int32, device=q8.device) if return_pv_count else None
+    pvc = torch.zeros((B, H, 4 * ((N + 127) // 128)), dtype=torch.int32, device=q8.device) if return_pv_count else None
     _check(load().spg_block_sparse_attn(_p(q8), _p(k8), _p(v8), _p(out), _dt(out), _p(lut), _p(valid), _p(pvthreshd),
                                         _p(q_scale), _p(k_scale), _p(v_scale), B, H, N, D, float(sm_scale),
                                         int(bool(is_causal)), _p(pvc), _stream()))
@@ -227,7 +227,7 @@ def block_sparse_attn_f16v(q8, k8, vt, out, lut, valid, pvthreshd, q_scale, k_sc
                            return_pv_count=False):
     _dev(q8, k8, vt, out, lut, valid, pvthreshd, q_scale, k_scale)
     B, H, N, D = q8.shape
-    pvc = torch.zeros((B, H, (N + 127) // 128), dtype=torch.int32, device=q8.device) if return_pv_count else None
+    pvc = torch.zeros((B, H, 4 * ((N + 127) // 128)), dtype=torch.int32, device=q8.device) if return_pv_count else None
     _check(load().spg_block_sparse_attn_f16v(_p(q8), _p(k8), _p(vt), _p(out), _dt(out), _p(lut), _p(valid),
                                              _p(pvthreshd), _p(q_scale), _p(k_scale), B, H, N, D, float(sm_scale),
                                              int(bool(is_causal)), _p(pvc), _stream()))

@@ -424,7 +424,9 @@ __global__ __launch_bounds__(256, PV16 ? 2 : 3) void block_sparse_attn_kernel(co
 #undef SPG_LOAD_TILES
 #undef SPG_LANE_OFFSETS
 
-  if (p.pv_count != nullptr && tid == 0) p.pv_count[(size_t)bh * p.nq + qb] = cnt;
+  // one count per wavefront of 32 query rows, the layout of the reference's PV_Count (sm89.cuh:650-659); the four
+  // counts of a Q block are equal because the skip decision is taken per block
+  if (p.pv_count != nullptr && lane == 0) p.pv_count[((size_t)bh * p.nq + qb) * 4 + wave] = cnt;
 
   // ---- epilogue: O / d * v_scale -> out dtype -----------------------------------------------------------
   const float dtot = PV16 ? dsum : half_swap_sum_f32(dsum);

@@ -52,7 +52,7 @@ def test_f16v_kernel_on_oracle_tensors(dtype, D, N, causal, topk):
     torch.cuda.synchronize()
     met = _check(out, res["out"])
     print(f"f16v {dtype} D{D} N{N} causal={causal} topk={topk}: {met}", flush=True)
-    assert np.array_equal(pvc.cpu().numpy(), res["pv_count"])
+    assert np.array_equal(pvc.view(B, H, -1, 4).cpu().numpy(), np.repeat(res["pv_count"][..., None], 4, axis=-1))
 
 
 def test_f16v_pv_threshold_skips_like_the_oracle():
