@@ -1,4 +1,4 @@
-"""Full-size GPU checks on the BASELINE configurations through size-independent properties.
+"""Full-size GPU checks on the four large benchmark configurations (cfg2-cfg5 of spargeattn_amd/workloads.py) through size-independent properties.
 
 The oracle is too slow at these sizes; instead each test checks invariants the algorithm fixes (row counts of the
 block map, LUT sortedness, quantisation round-trip bounds, code-range of the FP8 tensor, determinism) and compares
