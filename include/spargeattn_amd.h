@@ -88,16 +88,17 @@ int spg_v_quant_fp8(const void *v, uint8_t *v8, float *v_scale, int B, int H, in
  * replaces qk_int8_sv_f8_accum_f32_block_sparse_attn_inst_buf_fuse_v_scale_with_pv_threshold
  * (csrc/qattn/attn_cuda.h:61-76, csrc/qattn/qk_int_sv_f8_cuda_sm89.cu:197-390) with
  * tensor_layout = HND, qk_quant_gran = per-block, PV threshold per block.
- * q8,k8 int8 (B,H,N,D); v8 as produced by spg_v_quant_fp8; out (B,H,N,D) out_dtype;
- * lut/valid_block_num as above; pvthreshd (H,) float32; q_scale (B,H,nq), k_scale (B,H,nk),
- * v_scale (B,H,D) float32; pv_count (B,H,nq*4) int32 or NULL: number of K blocks
+ * q8 int8 (B,H,N,D); k8 int8 (B,Hkv,N,D); v8 as produced by spg_v_quant_fp8 for Hkv heads; out (B,H,N,D) out_dtype;
+ * lut/valid_block_num as above; pvthreshd (H,) float32; q_scale (B,H,nq), k_scale (B,Hkv,nk),
+ * v_scale (B,Hkv,D) float32; Hkv divides H: query head h reads K/V head h / (H / Hkv) (grouped-query attention,
+ * sm89.cu:310-314, sm89.cuh:118); Hkv = H is plain multi-head attention; pv_count (B,H,nq*4) int32 or NULL: number of K blocks
  * whose PV was computed, one entry per 32 query rows as in the reference (sm89.cu:331-334); entries of Q blocks with
  * valid_block_num == 0 are left untouched.
  * Row blocks with valid_block_num == 0 are left unwritten, as in the reference (sm89.cuh:232-235). */
 int spg_block_sparse_attn(const int8_t *q8, const int8_t *k8, const uint8_t *v8, void *out, int out_dtype,
                           const int32_t *lut, const int32_t *valid_block_num, const float *pvthreshd,
                           const float *q_scale, const float *k_scale, const float *v_scale,
-                          int B, int H, int N, int D, float sm_scale, int is_causal, int32_t *pv_count,
+                          int B, int H, int Hkv, int N, int D, float sm_scale, int is_causal, int32_t *pv_count,
                           void *stream);
 
 /* ---- SageAttention1-style variant: INT8 QK^T, FP16 PV.
@@ -113,7 +114,7 @@ int spg_v_tiles_f16(const void *v, void *vt, int B, int H, int N, int D, int dty
 int spg_block_sparse_attn_f16v(const int8_t *q8, const int8_t *k8, const void *vt, void *out, int out_dtype,
                                const int32_t *lut, const int32_t *valid_block_num, const float *pvthreshd,
                                const float *q_scale, const float *k_scale,
-                               int B, int H, int N, int D, float sm_scale, int is_causal, int32_t *pv_count,
+                               int B, int H, int Hkv, int N, int D, float sm_scale, int is_causal, int32_t *pv_count,
                                void *stream);
 
 /* ---- measurement comparator: dense FP16 flash attention on MFMA (no counterpart in the reference;

@@ -67,6 +67,7 @@ def block_sparse_attention(q8, k8, v8, lut, valid, pvthreshd, q_scale, k_scale, 
     k8 = np.asarray(k8)
     b_, h_, n, d_ = q8.shape
     nkv = k8.shape[2]
+    groups = h_ // k8.shape[1]            # grouped-query attention: K/V head = query head // groups (sm89.cuh:118)
     nq = (n + CTA_Q - 1) // CTA_Q
     vf = e4m3fn_to_f32(v8) if pv == "fp8" else np.asarray(v8, dtype=F32)
     offset = S_FP8_OFFSET if pv == "fp8" else F32(0.0)
@@ -77,6 +78,7 @@ def block_sparse_attention(q8, k8, v8, lut, valid, pvthreshd, q_scale, k_scale, 
     for b in range(b_):
         for h in range(h_):
             thr = F32(pvthreshd[h])
+            hk = h // groups
             for i in range(nq):
                 nv = int(valid[b, h, i])
                 if nv == 0:
@@ -97,10 +99,10 @@ def block_sparse_attention(q8, k8, v8, lut, valid, pvthreshd, q_scale, k_scale, 
                     c0 = int(j) * CTA_K
                     cols = max(0, min(CTA_K, nkv - c0))
                     kb = np.zeros((CTA_K, d_), dtype=np.float64)
-                    kb[:cols] = k8[b, h, c0:c0 + cols]
-                    vb = vf[b, h, c0:c0 + CTA_K]
+                    kb[:cols] = k8[b, hk, c0:c0 + cols]
+                    vb = vf[b, hk, c0:c0 + CTA_K]
                     s = (qb @ kb.T).astype(F32)                 # exact integers
-                    dq = F32(qs * F32(k_scale[b, h, j]))
+                    dq = F32(qs * F32(k_scale[b, hk, j]))
                     if it < nv - 2:
                         a = F32(c * dq)
                         m_blk = (s.max(axis=1) * a).astype(F32)
@@ -140,7 +142,7 @@ def block_sparse_attention(q8, k8, v8, lut, valid, pvthreshd, q_scale, k_scale, 
                 pv_count[b, h, i] = cnt
                 res = (o / dsum[:, None]).astype(F32)
                 if pv == "fp8":
-                    res = res * np.asarray(v_scale[b, h], dtype=F32)[None, :]
+                    res = res * np.asarray(v_scale[b, hk], dtype=F32)[None, :]
                 out[b, h, r0:r0 + rows] = round_to(res[:rows].astype(np.float64), out_dtype)
     if return_pv_count:
         return out, written, pv_count

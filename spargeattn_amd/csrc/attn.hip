@@ -44,7 +44,7 @@ struct AttnParams {
   const int32_t *lut, *valid;
   const float *pvthr, *q_scale, *k_scale, *v_scale;
   int32_t *pv_count;
-  int B, H, N, nq, nk;
+  int B, H, Hkv, N, nq, nk;
   float sm_scale_log2;
   int is_causal;
   int total_wg, wg_per_xcd;
@@ -108,6 +108,8 @@ __global__ __launch_bounds__(256, PV16 ? 2 : 3) void block_sparse_attn_kernel(co
   const int bh = L / p.nq;
   const int qb = p.nq - 1 - (L % p.nq);
   const int head = bh % p.H;
+  // grouped-query attention: H / Hkv consecutive query heads share one K/V head (sm89.cuh:118, head_id / num_kv_groups)
+  const int bhk = (bh / p.H) * p.Hkv + head / (p.H / p.Hkv);
   const int nv = p.valid[(size_t)bh * p.nq + qb];
   if (nv == 0) return;                                       // output rows stay unwritten (sm89.cuh:232-235)
   const int32_t *lut_row = p.lut + ((size_t)bh * p.nq + qb) * p.nk;
@@ -125,14 +127,14 @@ __global__ __launch_bounds__(256, PV16 ? 2 : 3) void block_sparse_attn_kernel(co
     if (q_row < N) qreg[ks] = *(const v4i *)(p.q8 + ((size_t)bh * N + q_row) * D + 32 * ks + 16 * hh);
   }
 
-  const int8_t *kbase = p.k8 + (size_t)bh * N * D;
-  const uint8_t *vbase = p.v8 + (size_t)bh * p.nk * (size_t)VTILE;
+  const int8_t *kbase = p.k8 + (size_t)bhk * N * D;
+  const uint8_t *vbase = p.v8 + (size_t)bhk * p.nk * (size_t)VTILE;
   // LUT and K scales are read through the constant address space: uniform addresses become scalar loads (SMEM),
   // which never touch the vector-memory counter the tile ring is synchronised with.
   typedef const __attribute__((address_space(4))) int32_t *c_i32_t;
   typedef const __attribute__((address_space(4))) float *c_f32_t;
   const c_i32_t lutc = (c_i32_t)(p.lut + ((size_t)bh * p.nq + qb) * p.nk);
-  const c_f32_t kscale = (c_f32_t)(p.k_scale + (size_t)bh * p.nk);
+  const c_f32_t kscale = (c_f32_t)(p.k_scale + (size_t)bhk * p.nk);
   const float qs = ((c_f32_t)p.q_scale)[(size_t)bh * p.nq + qb];
   const float c = p.sm_scale_log2;
   const float thr = ((c_f32_t)p.pvthr)[head];
@@ -433,7 +435,7 @@ __global__ __launch_bounds__(256, PV16 ? 2 : 3) void block_sparse_attn_kernel(co
   const float inv = __builtin_amdgcn_rcpf(dtot);
   if (q_row < N) {
     uint16_t *orow = (uint16_t *)p.out + ((size_t)bh * N + q_row) * D;
-    const float *vs = p.v_scale + (size_t)bh * D;
+    const float *vs = p.v_scale + (size_t)bhk * D;
 #pragma unroll
     for (int dt = 0; dt < NDT; dt++) {
 #pragma unroll
@@ -454,11 +456,12 @@ __global__ __launch_bounds__(256, PV16 ? 2 : 3) void block_sparse_attn_kernel(co
 hipError_t launch_block_sparse_attn(const int8_t *q8, const int8_t *k8, const uint8_t *v8, void *out, int out_dtype,
                                     const int32_t *lut, const int32_t *valid, const float *pvthreshd,
                                     const float *q_scale, const float *k_scale, const float *v_scale, int B, int H,
-                                    int N, int D, float sm_scale, int is_causal, int32_t *pv_count, hipStream_t st) {
+                                    int Hkv, int N, int D, float sm_scale, int is_causal, int32_t *pv_count,
+                                    hipStream_t st) {
   AttnParams p;
   p.q8 = q8; p.k8 = k8; p.v8 = v8; p.out = out; p.lut = lut; p.valid = valid; p.pvthr = pvthreshd;
   p.q_scale = q_scale; p.k_scale = k_scale; p.v_scale = v_scale; p.pv_count = pv_count;
-  p.B = B; p.H = H; p.N = N; p.nq = (N + 127) / 128; p.nk = (N + 63) / 64;
+  p.B = B; p.H = H; p.Hkv = Hkv; p.N = N; p.nq = (N + 127) / 128; p.nk = (N + 63) / 64;
   p.sm_scale_log2 = sm_scale * SPG_LOG2E;
   p.is_causal = is_causal;
   p.total_wg = p.nq * H * B;

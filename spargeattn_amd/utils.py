@@ -66,6 +66,10 @@ def get_block_map_meansim_fuse_quant(q, k, km=None, is_causal=False, BLKQ=128, B
         or (cdfthreshd is not None and topk is None), "Only one of cdfthreshd and topk can be set."
     _check_blocks(BLKQ, BLKK)
     H = q.size(1)
+    if k.size(1) != H:
+        # the reference's pooled-score matmul fails on mismatching head counts (utils.py:388)
+        raise RuntimeError(f"mask prediction needs as many K heads as Q heads (got {k.size(1)} and {H}); "
+                           "grouped-query attention is supported by block_sparse_sage2_attn_cuda only")
     simthreshd1 = hyperparameter_check(simthreshd1, H, q.device)
     if cdfthreshd is not None:
         cdfthreshd = hyperparameter_check(cdfthreshd, H, q.device)

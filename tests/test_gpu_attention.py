@@ -218,3 +218,20 @@ def test_operator_under_hip_graph_capture():
     g.replay()
     torch.cuda.synchronize()
     assert torch.equal(out, sa.spas_sage2_attn_meansim_topk_cuda(q.flip(2).contiguous(), k, v, topk=cfg.topk))
+
+
+@pytest.mark.parametrize("H,Hkv,D,dtype", [(4, 2, 64, torch.float16), (6, 1, 128, torch.bfloat16)])
+def test_custom_mask_operator_with_grouped_kv_heads(H, Hkv, D, dtype):
+    B, N = 2, 640
+    q = rand_T((B, H, N, D), dtype, 70)
+    k = rand_T((B, Hkv, N, D), dtype, 71, shift=0.3)
+    v = rand_T((B, Hkv, N, D), dtype, 72)
+    g = torch.Generator().manual_seed(5)
+    mask = (torch.rand((B, H, 5, 10), generator=g) < 0.5).to(torch.int32)
+    mask[:, :, torch.arange(5), 2 * torch.arange(5)] = 1
+    res = oapi.block_sparse_sage2_attn(to_np(q), to_np(k), to_np(v), mask.numpy(), tag_of(dtype), pvthreshd=3.0)
+    o, sparsity = sa.block_sparse_sage2_attn_cuda(q, k, v, mask_id=mask.cuda(), pvthreshd=3.0, return_sparsity=True)
+    assert o.shape == q.shape and abs(sparsity - res["sparsity"]) < 1e-6
+    _check_out(o, res["out"])
+    with pytest.raises(RuntimeError, match="as many K heads"):
+        sa.spas_sage2_attn_meansim_topk_cuda(q, k, v)

@@ -181,3 +181,20 @@ def test_f16v_denominator_uses_rounded_p():
     exact = 1.0 / (1.0 + (n - 1) * target)
     got = float(out[0, 0, 5, 3])
     assert abs(got - rounded) < 4e-4 < abs(got - exact), (got, rounded, exact)
+
+
+def test_gqa_equals_mha_with_repeated_kv_heads():
+    """Grouped-query attention: query head h reads K/V head h // (H / Hkv) (sm89.cuh:118).  With K/V heads repeated
+    the multi-head path must give the identical result (quantisation is per K/V head, so nothing else changes)."""
+    tag, d, n, H, Hkv = R.BF16, 64, 384, 4, 2
+    rng = np.random.default_rng(21)
+    mk = lambda h: R.round_to(rng.standard_normal((1, h, n, d)), tag)
+    q, k, v = mk(H), mk(Hkv) + 0.3, mk(Hkv)
+    mask = (rng.random((1, H, 3, 6)) < 0.5).astype(np.int32)
+    mask[:, :, np.arange(3), 2 * np.arange(3)] = 1
+    res = api.block_sparse_sage2_attn(q, k, v, mask, tag, pvthreshd=4.0)
+    rep = api.block_sparse_sage2_attn(q, np.repeat(k, H // Hkv, axis=1), np.repeat(v, H // Hkv, axis=1), mask, tag,
+                                      pvthreshd=4.0)
+    assert res["k8"].shape[1] == Hkv and rep["k8"].shape[1] == H
+    assert np.array_equal(res["out"], rep["out"]) and np.array_equal(res["pv_count"], rep["pv_count"])
+    assert not np.array_equal(res["out"][:, 0], res["out"][:, 2])       # heads of different groups do differ
