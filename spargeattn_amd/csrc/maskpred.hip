@@ -183,6 +183,12 @@ __global__ __launch_bounds__(256) void pool_sim_quant_kernel(const uint16_t *__r
     // rows.  Both are computed ONCE per NP rows - lane c of the group takes row c % NP - and handed round with lane
     // reads, instead of NP times in every lane.
     static_assert(NP <= TPR, "one lane of the row group per row");
+    // A NEGATIVE similarity threshold (the top-k operators' default, -0.1) decides the flag without the normalised rows:
+    // the statistic is ||sum of x_hat||^2 / rows^2 >= 0 > threshold whenever every x_hat is finite.  x_hat = x / norm is
+    // non-finite exactly for rows with norm == 0 (all-zero rows such as the padding of a partial block, or rows too
+    // small for their squares) and for non-finite x; |x| <= norm (1 + 2^-23) keeps every other quotient within fp16.
+    const bool sim_trivial = simthr[bh % H] < 0.f;     // workgroup-uniform
+    int bad_rows = 0;
     float ssf_mine = 0.f;
 #pragma unroll
     for (int p = 0; p < NP; p++) {
@@ -196,7 +202,15 @@ __global__ __launch_bounds__(256) void pool_sim_quant_kernel(const uint16_t *__r
       ss = group_sum_f64<TPR>(ss);                 // the TPR lanes of this row
       const float ssf = (float)ss;
       ssf_mine = (c % NP == p) ? ssf : ssf_mine;
+      if (sim_trivial) {
+        if (!(ssf < INFINITY)) {                     // overflow of finite values is harmless (x / inf = 0); inf or NaN x is not
+#pragma unroll
+          for (int e = 0; e < 8; e++) bad_rows |= __builtin_isfinite(xf[p][e]) ? 0 : 1;
+        }
+        bad_rows |= (ssf == 0.f) ? 1 : 0;
+      }
     }
+    if (!sim_trivial) {
     const float norm_mine = sqrtf(ssf_mine);
     const float rn_mine = rcp_safe(norm_mine) ? exact_rcp(norm_mine) : 0.f;
     const int group_lane0 = (tid & 63) & ~(TPR - 1);
@@ -218,15 +232,24 @@ __global__ __launch_bounds__(256) void pool_sim_quant_kernel(const uint16_t *__r
         }
       }
     }
+    }   // !sim_trivial
 #pragma unroll
-    for (int e = 0; e < 8; e++) { s_col[r][c * 8 + e] = colsum[e]; s_xh[r][c * 8 + e] = colxh[e]; }
+    for (int e = 0; e < 8; e++) s_col[r][c * 8 + e] = colsum[e];
+    if (!sim_trivial) {
+#pragma unroll
+      for (int e = 0; e < 8; e++) s_xh[r][c * 8 + e] = colxh[e];
+    }
     __syncthreads();
     long long g = 0;
-    int bad = 0;
+    int bad = bad_rows;
     if (tid < D) {
-      double s = 0.0, sx = 0.0;
-      for (int i = 0; i < RPP; i++) { s += s_col[i][tid]; sx += s_xh[i][tid]; }
+      double s = 0.0;
+      for (int i = 0; i < RPP; i++) s += s_col[i][tid];
       pool[((size_t)bh * nb + blk) * D + tid] = f64_to_elem<DT>(s / (double)rows_valid);
+    }
+    if (!sim_trivial && tid < D) {
+      double sx = 0.0;
+      for (int i = 0; i < RPP; i++) sx += s_xh[i][tid];
       if (__builtin_isfinite(sx)) {
         const long long si = (long long)(sx * 16777216.0);   // exact integer
         g = si * si;
@@ -241,7 +264,7 @@ __global__ __launch_bounds__(256) void pool_sim_quant_kernel(const uint16_t *__r
     if (tid == 0) {
       const long long gt = s_wg[0] + s_wg[1] + s_wg[2] + s_wg[3];   // = sum(gram) * 2^48, exact
       const double thr = (double)simthr[bh % H] * (double)(rows_valid * rows_valid) * 281474976710656.0;
-      sim[(size_t)bh * nb + blk] = (!any_bad && (double)gt > thr) ? 1 : 0;
+      sim[(size_t)bh * nb + blk] = (!any_bad && (sim_trivial || (double)gt > thr)) ? 1 : 0;
     }
   } else {
     __syncthreads();

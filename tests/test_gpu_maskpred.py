@@ -135,3 +135,36 @@ def test_shared_reciprocal_division_is_ieee():
     for seed in (1, 2):
         total, bad = _lib.selftest_division(1 << 18, seed)
         assert total > (1 << 18) * 100000 and bad == 0, (seed, total, bad)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("thr_value", [-0.1, -1.0, 0.0, 0.3])
+def test_similarity_flag_on_degenerate_rows(dtype, thr_value):
+    """Negative thresholds are decided without the normalised rows; the flag must still match the oracle on all-zero
+    rows, rows whose squares underflow, rows whose squares overflow binary32, infinities and NaNs."""
+    B, H, N, D = 1, 2, 128 * 8, 64
+    tag = tag_of(dtype)
+    x = rand_T((B, H, N, D), dtype, 9)
+    big = 3.0e38 if dtype == torch.bfloat16 else 60000.0
+    tiny = 1.0e-30 if dtype == torch.bfloat16 else 6.0e-8
+    x[0, 0, 128 * 1 + 5] = 0                      # an all-zero row          -> block 1 not similar
+    x[0, 0, 128 * 2 + 7] = tiny                   # squares underflow        -> block 2: norm 0 in binary32 (bf16 only)
+    x[0, 0, 128 * 3 + 9] = big                    # sum of squares overflows binary32 (bf16): x / inf = 0, still finite
+    x[0, 0, 128 * 4 + 11, 3] = float("inf")       # -> not similar
+    x[0, 0, 128 * 5 + 13, 60] = float("nan")      # -> not similar
+    x[0, 1, 128 * 6 + 1, :32] = 0                 # half a row of zeros is harmless
+    thr = torch.tensor([thr_value] * H, dtype=torch.float32, device="cuda")
+    for bs in (128, 64):
+        pool, sim, xq, scale = _lib.pool_sim_quant(x, None, bs, thr)
+        ref = mp.pool_sim_quant(to_np(x), None, bs, thr.cpu().numpy(), tag)
+        assert np.array_equal(sim.cpu().numpy(), ref["sim"]), (bs, sim.cpu().numpy(), ref["sim"])
+    if thr_value < 0:
+        want = np.ones((1, 2, 8), bool)
+        want[0, 0, [1, 4, 5]] = False
+        if dtype == torch.bfloat16:
+            want[0, 0, 2] = False
+        assert np.array_equal(ref_sim_128(x, thr, tag), want)
+
+
+def ref_sim_128(x, thr, tag):
+    return mp.pool_sim_quant(to_np(x), None, 128, thr.cpu().numpy(), tag)["sim"]
