@@ -208,6 +208,38 @@ def main():
                              + (" for QK^T and dense fp16 MFMA for PV, blended" if sage1 else "")},
     }
 
+    # ---- accuracy of the operator output on sampled Q blocks: against dense fp32 attention on the original tensors
+    #      (includes the effect of dropping blocks) and against fp32 attention restricted to the selected blocks -------
+    o = step()
+    km = _lib.km_mean(k)
+    lut, valid, *_ = utils.get_block_map_meansim_fuse_quant(q, k, km, is_causal=cfg.is_causal, simthreshd1=-0.1,
+                                                            cdfthreshd=None, topk=cfg.topk, return_lut=True)
+    num = {"dense": [0.0, 0.0, 0.0, 0.0, 0.0], "masked": [0.0, 0.0, 0.0, 0.0, 0.0]}
+    samples = [(0, nq // 2), (H // 2, nq - 1), (H - 1, nq // 5)]
+    for (h, qb) in samples:
+        r0, r1 = qb * 128, min(N, qb * 128 + 128)
+        sc = (q[0, h, r0:r1].float() @ k[0, h].float().T) * D ** -0.5
+        if cfg.is_causal:
+            rows = torch.arange(r0, r1, device=dev)[:, None]
+            sc = sc.masked_fill(torch.arange(N, device=dev)[None, :] > rows, float("-inf"))
+        idx = torch.cumsum(lut[0, h, qb, :int(valid[0, h, qb])].long(), 0)
+        bm = torch.zeros(nk, dtype=torch.bool, device=dev)
+        bm[idx] = True
+        tok = bm.repeat_interleave(64)[:N]
+        got = o[0, h, r0:r1].float()
+        for name, scores in (("dense", sc), ("masked", sc.masked_fill(~tok[None, :], float("-inf")))):
+            ref = torch.softmax(scores, dim=-1) @ v[0, h].float()
+            a = num[name]
+            a[0] += float((got * ref).sum()); a[1] += float((got * got).sum()); a[2] += float((ref * ref).sum())
+            a[3] += float((got - ref).abs().sum()); a[4] += float(ref.abs().sum())
+    out["accuracy"] = {
+        "sample": f"Q blocks {samples} (head, block) of batch 0",
+        "vs_fp32_attention_on_selected_blocks": {"cos": num["masked"][0] / (num["masked"][1] * num["masked"][2]) ** 0.5,
+                                                 "rel_l1": num["masked"][3] / num["masked"][4]},
+        "vs_dense_fp32_sdpa": {"cos": num["dense"][0] / (num["dense"][1] * num["dense"][2]) ** 0.5,
+                               "rel_l1": num["dense"][3] / num["dense"][4]}}
+    del o, lut, valid, km
+
     if not args.no_dense:
         qh, kh, vh = q.to(torch.float16), k.to(torch.float16), v.to(torch.float16)
         vt = _lib.v_tiles_f16(vh)
