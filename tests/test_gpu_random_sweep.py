@@ -15,21 +15,21 @@ pytestmark = pytest.mark.gpu
 def _cases():
     rng = np.random.default_rng(20240607)
     out = []
-    for i in range(14):
+    for i in range(40):
         D = int(rng.choice([64, 128]))
         dtype = [torch.float16, torch.bfloat16][int(rng.integers(2))]
         B, H = int(rng.integers(1, 3)), int(rng.integers(1, 4))
-        N = int(rng.integers(128, 1300))
+        N = int(rng.choice([128, 129, 191, 193, 255, 257, 511, 513, 1023, 1025, int(rng.integers(128, 1300))]))
         causal = bool(rng.integers(2))
         mode = ["topk", "cdf"][int(rng.integers(2))]
         out.append((i, B, H, N, D, dtype, causal, mode, float(rng.uniform(0.2, 0.9)), bool(rng.integers(2)),
-                    float(rng.choice([50.0, 3.0, 0.5]))))
+                    float(rng.choice([50.0, 3.0, 0.5])), float(rng.choice([-0.1, 0.0, 0.3, 0.8]))))
     return out
 
 
 @pytest.mark.parametrize("case", _cases(), ids=lambda c: f"{c[0]}-B{c[1]}H{c[2]}N{c[3]}D{c[4]}-{'c' if c[6] else 'n'}-{c[7]}")
 def test_random_case(case):
-    i, B, H, N, D, dtype, causal, mode, level, sink, pvthr = case
+    i, B, H, N, D, dtype, causal, mode, level, sink, pvthr, sim = case
     g = torch.Generator().manual_seed(1000 + i)
     base = torch.randn((B, H, 1, D), generator=g)
     q = (torch.randn((B, H, N, D), generator=g) + 0.5 * base).to(dtype)
@@ -39,7 +39,6 @@ def test_random_case(case):
     n0 = N // 3
     q[:, :, :n0] = (q[:, :, :1] + 0.05 * q[:, :, :n0].float()).to(dtype)
     kw = dict(topk=level, cdfthreshd=None) if mode == "topk" else dict(topk=None, cdfthreshd=level)
-    sim = 0.3
     res = oapi.spas_sage2_attn_meansim_topk(to_np(q), to_np(k), to_np(v), tag_of(dtype), is_causal=causal,
                                             simthreshd1=sim, pvthreshd=pvthr, attention_sink=sink, **kw)
     qg, kg, vg = q.cuda(), k.cuda(), v.cuda()
