@@ -33,6 +33,11 @@ enum spg_status {
 
 enum spg_dtype { SPG_F16 = 0, SPG_BF16 = 1 };
 
+/* PVThresholdMode of the reference (csrc/qattn/attn_utils.cuh:58-62): whether the P.V product of a K block is skipped
+ * when no row's running maximum came within pvthreshd of being raised by it - never, decided for the whole 128-row
+ * Q block (the mode every Python entry point of the reference uses), or for each 32 query rows on their own. */
+enum spg_pv_threshold_mode { SPG_PV_NONE = 0, SPG_PV_PER_BLOCK = 1, SPG_PV_PER_WARP = 2 };
+
 /* element kinds accepted for a user block mask ("non-zero = keep", spas_sage_attn/utils.py:68-69) */
 enum spg_mask_kind {
   SPG_MASK_I8 = 0, SPG_MASK_I16 = 1, SPG_MASK_I32 = 2, SPG_MASK_I64 = 3,
@@ -87,7 +92,8 @@ int spg_v_quant_fp8(const void *v, uint8_t *v8, float *v_scale, int B, int H, in
 /* ---- A11: block-sparse INT8-QK / FP8-PV attention ------------------------------------------------
  * replaces qk_int8_sv_f8_accum_f32_block_sparse_attn_inst_buf_fuse_v_scale_with_pv_threshold
  * (csrc/qattn/attn_cuda.h:61-76, csrc/qattn/qk_int_sv_f8_cuda_sm89.cu:197-390) with
- * tensor_layout = HND, qk_quant_gran = per-block, PV threshold per block.
+ * tensor_layout = HND, qk_quant_gran = per-block; pv_threshold_mode = SPG_PV_PER_BLOCK is what that entry point
+ * compiles in (sm89.cu:365), the other two modes are the kernel template's (sm89.cuh:283-391).
  * q8 int8 (B,H,N,D); k8 int8 (B,Hkv,N,D); v8 as produced by spg_v_quant_fp8 for Hkv heads; out (B,H,N,D) out_dtype;
  * lut/valid_block_num as above; pvthreshd (H,) float32; q_scale (B,H,nq), k_scale (B,Hkv,nk),
  * v_scale (B,Hkv,D) float32; Hkv divides H: query head h reads K/V head h / (H / Hkv) (grouped-query attention,
@@ -98,8 +104,8 @@ int spg_v_quant_fp8(const void *v, uint8_t *v8, float *v_scale, int B, int H, in
 int spg_block_sparse_attn(const int8_t *q8, const int8_t *k8, const uint8_t *v8, void *out, int out_dtype,
                           const int32_t *lut, const int32_t *valid_block_num, const float *pvthreshd,
                           const float *q_scale, const float *k_scale, const float *v_scale,
-                          int B, int H, int Hkv, int N, int D, float sm_scale, int is_causal, int32_t *pv_count,
-                          void *stream);
+                          int B, int H, int Hkv, int N, int D, float sm_scale, int is_causal, int pv_threshold_mode,
+                          int32_t *pv_count, void *stream);
 
 /* ---- SageAttention1-style variant: INT8 QK^T, FP16 PV.
  * Replaces qk_int8_sv_f16_accum_f16_block_sparse_attn_inst_buf_with_pv_threshold (csrc/qattn/attn_cuda.h:32-45,
@@ -114,8 +120,8 @@ int spg_v_tiles_f16(const void *v, void *vt, int B, int H, int N, int D, int dty
 int spg_block_sparse_attn_f16v(const int8_t *q8, const int8_t *k8, const void *vt, void *out, int out_dtype,
                                const int32_t *lut, const int32_t *valid_block_num, const float *pvthreshd,
                                const float *q_scale, const float *k_scale,
-                               int B, int H, int Hkv, int N, int D, float sm_scale, int is_causal, int32_t *pv_count,
-                               void *stream);
+                               int B, int H, int Hkv, int N, int D, float sm_scale, int is_causal, int pv_threshold_mode,
+                               int32_t *pv_count, void *stream);
 
 /* ---- measurement comparator: dense FP16 flash attention on MFMA (no counterpart in the reference;
  * the "dense FP16 attention kernel built in the same run" the speed-up is quoted against).

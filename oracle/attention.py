@@ -47,11 +47,14 @@ def _fma(a, b, c):
 
 
 def block_sparse_attention(q8, k8, v8, lut, valid, pvthreshd, q_scale, k_scale, v_scale,
-                           sm_scale, out_dtype, is_causal=False, return_pv_count=False, pv="fp8"):
+                           sm_scale, out_dtype, is_causal=False, return_pv_count=False, pv="fp8", pv_mode=1):
     """q8,k8 int8 (B,H,N,D); v8 e4m3 codes uint8 (B,H,Npad,D); lut/valid int32.
 
     Returns (out float32 (B,H,N,D) holding out_dtype values, written (B,H,nq) bool[, pv_count (B,H,nq)]).
     Row blocks with valid == 0 are left untouched (zeros here; sm89.cuh:232-235).
+    ``pv_mode`` is the kernel template's PVThresholdMode (attn_utils.cuh:58-62): 1 = the skip is decided for the whole
+    128-row block (what every Python entry point uses), 2 = for each warp of 32 rows on its own (sm89.cuh:302-318
+    without the block reduction of 320-343; pv_count is then (B,H,nq,4)), 0 = never skip.
 
     ``pv="f16"`` restates the SageAttention1 kernel instead (qk_int_sv_f16_cuda_sm80.cuh:42-671 instantiated with
     per-block quantisation, per-block PV threshold and the row sum on the tensor cores, sm80.cuh:690): ``v8`` then holds
@@ -62,7 +65,7 @@ def block_sparse_attention(q8, k8, v8, lut, valid, pvthreshd, q_scale, k_scale, 
     the block to its binary32 accumulator (compute_fp16_sv_permuted_inst_buf, attn_utils.cuh:683-751) - parity
     unpinned for that rounding, the comparison is by tolerance.
     """
-    assert pv in ("fp8", "f16")
+    assert pv in ("fp8", "f16") and pv_mode in (0, 1, 2)
     q8 = np.asarray(q8)
     k8 = np.asarray(k8)
     b_, h_, n, d_ = q8.shape
@@ -74,7 +77,7 @@ def block_sparse_attention(q8, k8, v8, lut, valid, pvthreshd, q_scale, k_scale, 
     c = F32(F32(sm_scale) * LOG2E)
     out = np.zeros((b_, h_, n, d_), dtype=F32)
     written = np.zeros((b_, h_, nq), dtype=bool)
-    pv_count = np.zeros((b_, h_, nq), dtype=np.int32)
+    pv_count = np.zeros((b_, h_, nq, 4), dtype=np.int32)
     for b in range(b_):
         for h in range(h_):
             thr = F32(pvthreshd[h])
@@ -94,7 +97,7 @@ def block_sparse_attention(q8, k8, v8, lut, valid, pvthreshd, q_scale, k_scale, 
                 o = np.zeros((CTA_Q, d_), dtype=F32)
                 idxs = np.cumsum(lut[b, h, i, :nv].astype(np.int64))
                 qs = F32(q_scale[b, h, i])
-                cnt = 0
+                cnt = np.zeros(4, dtype=np.int32)
                 for it, j in enumerate(idxs):
                     c0 = int(j) * CTA_K
                     cols = max(0, min(CTA_K, nkv - c0))
@@ -106,17 +109,24 @@ def block_sparse_attention(q8, k8, v8, lut, valid, pvthreshd, q_scale, k_scale, 
                     if it < nv - 2:
                         a = F32(c * dq)
                         m_blk = (s.max(axis=1) * a).astype(F32)
-                        delta = np.max((m_blk - m).astype(F32))
+                        d_row = (m_blk - m).astype(F32)
+                        if pv_mode == 1:
+                            act4 = np.full(4, bool(F32(np.max(d_row) + thr) > 0))
+                        elif pv_mode == 2:
+                            act4 = (d_row.reshape(4, 32).max(axis=1) + thr).astype(F32) > 0
+                        else:
+                            act4 = np.ones(4, dtype=bool)
                         m_new = np.maximum(m, m_blk)
                         o_scale = _exp2(m - m_new)
                         dsum = (dsum * o_scale).astype(F32)
                         o = (o * o_scale[:, None]).astype(F32)
                         m = m_new
-                        if not (F32(delta + thr) > 0):
+                        if not act4.any():
                             continue
                         neg_m = (-m + offset).astype(F32)
                         p = _exp2(_fma(s, a, neg_m[:, None]))
                     else:
+                        act4 = np.ones(4, dtype=bool)
                         sf = (s * dq).astype(F32)
                         k_idx = c0 + np.arange(CTA_K)
                         if is_causal:
@@ -131,21 +141,22 @@ def block_sparse_attention(q8, k8, v8, lut, valid, pvthreshd, q_scale, k_scale, 
                         m = m_new
                         neg_m = (-m + offset).astype(F32)
                         p = _exp2(_fma(sf, c, neg_m[:, None]))
-                    cnt += 1
+                    cnt += act4
+                    act = np.repeat(act4, 32)
                     if pv == "fp8":
-                        dsum = (dsum + p.sum(axis=1, dtype=F32)).astype(F32)
+                        dsum = np.where(act, (dsum + p.sum(axis=1, dtype=F32)).astype(F32), dsum)
                         p8 = e4m3fn_to_f32(f32_to_e4m3fn(p))
                     else:
                         p8 = round_to(p.astype(np.float64), "fp16").astype(F32)
-                        dsum = (dsum + p8.sum(axis=1, dtype=F32)).astype(F32)
-                    o = (o + (p8 @ vb).astype(F32)).astype(F32)
+                        dsum = np.where(act, (dsum + p8.sum(axis=1, dtype=F32)).astype(F32), dsum)
+                    o = np.where(act[:, None], (o + (p8 @ vb).astype(F32)).astype(F32), o)
                 pv_count[b, h, i] = cnt
                 res = (o / dsum[:, None]).astype(F32)
                 if pv == "fp8":
                     res = res * np.asarray(v_scale[b, hk], dtype=F32)[None, :]
                 out[b, h, r0:r0 + rows] = round_to(res[:rows].astype(np.float64), out_dtype)
     if return_pv_count:
-        return out, written, pv_count
+        return out, written, (pv_count if pv_mode == 2 else pv_count[..., 0])
     return out, written
 
 

@@ -29,9 +29,9 @@ SIGNATURES = {
     "spg_block_select": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp]),
     "spg_map_to_lut": (_i, [_vp, _i, _vp, _vp, _i, _i, _i, _i, _vp]),
     "spg_v_quant_fp8": (_i, [_vp, _vp, _vp, _i, _i, _i, _i, _i, _vp]),
-    "spg_block_sparse_attn": (_i, [_vp, _vp, _vp, _vp, _i, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _f, _i, _vp, _vp]),
+    "spg_block_sparse_attn": (_i, [_vp, _vp, _vp, _vp, _i, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _f, _i, _i, _vp, _vp]),
     "spg_v_tiles_f16": (_i, [_vp, _vp, _i, _i, _i, _i, _i, _vp]),
-    "spg_block_sparse_attn_f16v": (_i, [_vp] * 4 + [_i] + [_vp] * 5 + [_i] * 5 + [_f, _i, _vp, _vp]),
+    "spg_block_sparse_attn_f16v": (_i, [_vp] * 4 + [_i] + [_vp] * 5 + [_i] * 5 + [_f, _i, _i, _vp, _vp]),
     "spg_dense_attn_f16": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _f, _i, _vp]),
     "spg_selftest_division": (_i, [_vp, _i, ctypes.c_uint, _vp]),
 }
@@ -192,14 +192,17 @@ def v8_natural_to_tiles(v8_nat):
     return sw.reshape(B, H, nk, D, 64).contiguous()
 
 
+PV_NONE, PV_PER_BLOCK, PV_PER_WARP = 0, 1, 2
+
+
 def block_sparse_attn(q8, k8, v8, out, lut, valid, pvthreshd, q_scale, k_scale, v_scale, sm_scale,
-                      is_causal=False, return_pv_count=False):
+                      is_causal=False, return_pv_count=False, pv_mode=PV_PER_BLOCK):
     _dev(q8, k8, v8, out, lut, valid, pvthreshd, q_scale, k_scale, v_scale)
     B, H, N, D = q8.shape
     pvc = torch.zeros((B, H, 4 * ((N + 127) // 128)), dtype=torch.int32, device=q8.device) if return_pv_count else None
     _check(load().spg_block_sparse_attn(_p(q8), _p(k8), _p(v8), _p(out), _dt(out), _p(lut), _p(valid), _p(pvthreshd),
                                         _p(q_scale), _p(k_scale), _p(v_scale), B, H, k8.shape[1], N, D, float(sm_scale),
-                                        int(bool(is_causal)), _p(pvc), _stream()))
+                                        int(bool(is_causal)), int(pv_mode), _p(pvc), _stream()))
     return pvc
 
 
@@ -224,13 +227,13 @@ def v_tiles_f16_to_natural(vt):
 
 
 def block_sparse_attn_f16v(q8, k8, vt, out, lut, valid, pvthreshd, q_scale, k_scale, sm_scale, is_causal=False,
-                           return_pv_count=False):
+                           return_pv_count=False, pv_mode=PV_PER_BLOCK):
     _dev(q8, k8, vt, out, lut, valid, pvthreshd, q_scale, k_scale)
     B, H, N, D = q8.shape
     pvc = torch.zeros((B, H, 4 * ((N + 127) // 128)), dtype=torch.int32, device=q8.device) if return_pv_count else None
     _check(load().spg_block_sparse_attn_f16v(_p(q8), _p(k8), _p(vt), _p(out), _dt(out), _p(lut), _p(valid),
                                              _p(pvthreshd), _p(q_scale), _p(k_scale), B, H, k8.shape[1], N, D, float(sm_scale),
-                                             int(bool(is_causal)), _p(pvc), _stream()))
+                                             int(bool(is_causal)), int(pv_mode), _p(pvc), _stream()))
     return pvc
 
 

@@ -47,6 +47,7 @@ struct AttnParams {
   int B, H, Hkv, N, nq, nk;
   float sm_scale_log2;
   int is_causal;
+  int pv_mode;     // PVThresholdMode of the reference (attn_utils.cuh:58-62): 0 none, 1 per block, 2 per wavefront of 32 rows
   int total_wg, wg_per_xcd;
 };
 
@@ -293,16 +294,19 @@ __global__ __launch_bounds__(256, PV16 ? 2 : 3) void block_sparse_attn_kernel(co
     const float m_new = fmaxf(m, fm);
     const float osc = __builtin_amdgcn_exp2f(m - m_new);
     m = m_new;
+    int vote = 1;
     if (!tail) {
       // max over rows of (diff) + thr > 0  <=>  some row has diff + thr > 0 (fp32 addition is monotonic)
-      const int vote = __any(diff + thr > 0.f);
+      vote = __any(diff + thr > 0.f);
       if (lane == 0) sVote[it & 1][wave] = vote;
     }
     __builtin_amdgcn_s_waitcnt(0x0F70);   // this wave's share of block it+1's tiles has landed in LDS
     __syncthreads();   // block it+1's tiles are complete; the votes are visible; ring slot of block it-1 is free
     bool compute = true;
-    if (!tail)         // workgroup-uniform (PVThresholdMode::kPerBlock, sm89.cuh:318-353)
-      compute = (sVote[it & 1][0] | sVote[it & 1][1] | sVote[it & 1][2] | sVote[it & 1][3]) != 0;
+    if (!tail) {       // workgroup-uniform in the per-block mode (sm89.cuh:318-353), wavefront-uniform otherwise
+      const bool any_wave = (sVote[it & 1][0] | sVote[it & 1][1] | sVote[it & 1][2] | sVote[it & 1][3]) != 0;
+      compute = p.pv_mode == 1 ? any_wave : (p.pv_mode == 2 ? vote != 0 : true);
+    }
     if (it + 2 < nv) {
       const uint32_t b2 = bufoff == 0 ? 2 * TILE : bufoff - TILE;   // slot (it+2) % 3
       SPG_LOAD_TILES(blk2, b2);
@@ -456,14 +460,15 @@ __global__ __launch_bounds__(256, PV16 ? 2 : 3) void block_sparse_attn_kernel(co
 hipError_t launch_block_sparse_attn(const int8_t *q8, const int8_t *k8, const uint8_t *v8, void *out, int out_dtype,
                                     const int32_t *lut, const int32_t *valid, const float *pvthreshd,
                                     const float *q_scale, const float *k_scale, const float *v_scale, int B, int H,
-                                    int Hkv, int N, int D, float sm_scale, int is_causal, int32_t *pv_count,
-                                    hipStream_t st) {
+                                    int Hkv, int N, int D, float sm_scale, int is_causal, int pv_mode,
+                                    int32_t *pv_count, hipStream_t st) {
   AttnParams p;
   p.q8 = q8; p.k8 = k8; p.v8 = v8; p.out = out; p.lut = lut; p.valid = valid; p.pvthr = pvthreshd;
   p.q_scale = q_scale; p.k_scale = k_scale; p.v_scale = v_scale; p.pv_count = pv_count;
   p.B = B; p.H = H; p.Hkv = Hkv; p.N = N; p.nq = (N + 127) / 128; p.nk = (N + 63) / 64;
   p.sm_scale_log2 = sm_scale * SPG_LOG2E;
   p.is_causal = is_causal;
+  p.pv_mode = pv_mode;
   p.total_wg = p.nq * H * B;
   p.wg_per_xcd = (p.total_wg + 7) / 8;
   const int grid = p.wg_per_xcd * 8;

@@ -38,6 +38,12 @@ int check_kv_heads(const char *fn, int H, int Hkv) {
   return SPG_OK;
 }
 
+int check_pv_mode(const char *fn, int mode) {
+  if (mode < SPG_PV_NONE || mode > SPG_PV_PER_WARP)
+    return fail(SPG_ERR_INVALID, "%s: pv_threshold_mode must be 0 (none), 1 (per block) or 2 (per 32 query rows), got %d", fn, mode);
+  return SPG_OK;
+}
+
 int check_dtype(const char *fn, int dtype) {
   if (dtype != SPG_F16 && dtype != SPG_BF16) return fail(SPG_ERR_INVALID, "%s: dtype must be SPG_F16 or SPG_BF16 (got %d)", fn, dtype);
   return SPG_OK;
@@ -129,17 +135,18 @@ int spg_v_quant_fp8(const void *v, uint8_t *v8, float *v_scale, int B, int H, in
 int spg_block_sparse_attn(const int8_t *q8, const int8_t *k8, const uint8_t *v8, void *out, int out_dtype,
                           const int32_t *lut, const int32_t *valid_block_num, const float *pvthreshd,
                           const float *q_scale, const float *k_scale, const float *v_scale, int B, int H, int Hkv, int N,
-                          int D, float sm_scale, int is_causal, int32_t *pv_count, void *stream) {
+                          int D, float sm_scale, int is_causal, int pv_threshold_mode, int32_t *pv_count, void *stream) {
   const char *fn = "spg_block_sparse_attn";
   SPG_TRY(check_shape(fn, B, H, N, D));
   SPG_TRY(check_kv_heads(fn, H, Hkv));
+  SPG_TRY(check_pv_mode(fn, pv_threshold_mode));
   SPG_TRY(check_dtype(fn, out_dtype));
   SPG_NONNULL(fn, q8); SPG_NONNULL(fn, k8); SPG_NONNULL(fn, v8); SPG_NONNULL(fn, out); SPG_NONNULL(fn, lut);
   SPG_NONNULL(fn, valid_block_num); SPG_NONNULL(fn, pvthreshd); SPG_NONNULL(fn, q_scale); SPG_NONNULL(fn, k_scale);
   SPG_NONNULL(fn, v_scale);
   return check_launch(fn, spg::launch_block_sparse_attn(q8, k8, v8, out, out_dtype, lut, valid_block_num, pvthreshd,
                                                         q_scale, k_scale, v_scale, B, H, Hkv, N, D, sm_scale,
-                                                        is_causal ? 1 : 0, pv_count, (hipStream_t)stream));
+                                                        is_causal ? 1 : 0, pv_threshold_mode, pv_count, (hipStream_t)stream));
 }
 
 int spg_v_tiles_f16(const void *v, void *vt, int B, int H, int N, int D, int dtype, void *stream) {
@@ -154,16 +161,17 @@ int spg_v_tiles_f16(const void *v, void *vt, int B, int H, int N, int D, int dty
 int spg_block_sparse_attn_f16v(const int8_t *q8, const int8_t *k8, const void *vt, void *out, int out_dtype,
                                const int32_t *lut, const int32_t *valid_block_num, const float *pvthreshd,
                                const float *q_scale, const float *k_scale, int B, int H, int Hkv, int N, int D,
-                               float sm_scale, int is_causal, int32_t *pv_count, void *stream) {
+                               float sm_scale, int is_causal, int pv_threshold_mode, int32_t *pv_count, void *stream) {
   const char *fn = "spg_block_sparse_attn_f16v";
   SPG_TRY(check_shape(fn, B, H, N, D));
   SPG_TRY(check_kv_heads(fn, H, Hkv));
+  SPG_TRY(check_pv_mode(fn, pv_threshold_mode));
   SPG_TRY(check_dtype(fn, out_dtype));
   SPG_NONNULL(fn, q8); SPG_NONNULL(fn, k8); SPG_NONNULL(fn, vt); SPG_NONNULL(fn, out); SPG_NONNULL(fn, lut);
   SPG_NONNULL(fn, valid_block_num); SPG_NONNULL(fn, pvthreshd); SPG_NONNULL(fn, q_scale); SPG_NONNULL(fn, k_scale);
   return check_launch(fn, spg::launch_block_sparse_attn(q8, k8, (const uint8_t *)vt, out, out_dtype, lut, valid_block_num,
                                                         pvthreshd, q_scale, k_scale, nullptr, B, H, Hkv, N, D, sm_scale,
-                                                        is_causal ? 1 : 0, pv_count, (hipStream_t)stream));
+                                                        is_causal ? 1 : 0, pv_threshold_mode, pv_count, (hipStream_t)stream));
 }
 
 int spg_dense_attn_f16(const void *q, const void *k, const void *v, void *out, int B, int H, int N, int D,

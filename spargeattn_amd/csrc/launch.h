@@ -26,8 +26,8 @@ void launch_v_tiles_f16(const void *v, void *vt, int B, int H, int N, int D, int
 hipError_t launch_block_sparse_attn(const int8_t *q8, const int8_t *k8, const uint8_t *v8, void *out, int out_dtype,
                                     const int32_t *lut, const int32_t *valid, const float *pvthreshd,
                                     const float *q_scale, const float *k_scale, const float *v_scale, int B, int H,
-                                    int Hkv, int N, int D, float sm_scale, int is_causal, int32_t *pv_count,
-                                    hipStream_t st);
+                                    int Hkv, int N, int D, float sm_scale, int is_causal, int pv_mode,
+                                    int32_t *pv_count, hipStream_t st);
 
 hipError_t launch_dense_attn_f16(const void *q, const void *k, const void *v, void *out, int B, int H, int N, int D,
                                  float sm_scale, int is_causal, hipStream_t st);

@@ -60,5 +60,7 @@ def test_argument_errors_are_reported_without_a_gpu():
     rc = lib.spg_v_quant_fp8(1, 1, 1, 1, 1, 128, 64, 7, None)
     assert rc == _lib.SPG_ERR_INVALID and b"dtype" in lib.spg_last_error()
     assert lib.spg_km_mean_workspace_bytes(1, 32, 32768, 128) > 0
-    rc = lib.spg_block_sparse_attn(1, 1, 1, 1, 0, 1, 1, 1, 1, 1, 1, 1, 6, 4, 128, 64, 0.125, 0, None, None)
+    rc = lib.spg_block_sparse_attn(1, 1, 1, 1, 0, 1, 1, 1, 1, 1, 1, 1, 6, 4, 128, 64, 0.125, 0, 1, None, None)
     assert rc == _lib.SPG_ERR_INVALID and b"must be divisible by num_kv_heads" in lib.spg_last_error()
+    rc = lib.spg_block_sparse_attn(1, 1, 1, 1, 0, 1, 1, 1, 1, 1, 1, 1, 4, 4, 128, 64, 0.125, 0, 3, None, None)
+    assert rc == _lib.SPG_ERR_INVALID and b"pv_threshold_mode" in lib.spg_last_error()

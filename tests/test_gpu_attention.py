@@ -235,3 +235,48 @@ def test_custom_mask_operator_with_grouped_kv_heads(H, Hkv, D, dtype):
     _check_out(o, res["out"])
     with pytest.raises(RuntimeError, match="as many K heads"):
         sa.spas_sage2_attn_meansim_topk_cuda(q, k, v)
+
+
+@pytest.mark.parametrize("fp16v", [False, True])
+def test_pv_threshold_modes_match_the_oracle(fp16v):
+    """Per-block (the API's), per-32-rows and no PV threshold: outputs and the per-wavefront PV counts."""
+    d, nblk = 64, 6
+    n = 64 * nblk
+    rng = np.random.default_rng(5)
+    nqb = n // 128                                           # queries and keys share one sequence length at this boundary
+    q8 = rng.integers(-20, 21, size=(1, 1, n, d)).astype(np.int8)
+    k8 = rng.integers(-20, 21, size=(1, 1, n, d)).astype(np.int8)
+    q8[0, 0, 32:64, 0] = 120
+    k8[0, 0, :64, 0] = 120                                   # block 0 dominates for rows 32..63 only
+    lut = np.ones((1, 1, nqb, nblk), np.int32); lut[..., 0] = 0
+    valid = np.full((1, 1, nqb), nblk, np.int32)
+    # scales small enough that no row is dominated by a few keys (the e4m3 rounding of P then averages out), while block 0
+    # still beats every other block by about one unit of log2 for rows 32..63
+    qs = np.full((1, 1, nqb), 0.02, np.float32); ks = np.full((1, 1, nblk), 0.02, np.float32)
+    thr = np.array([0.25], np.float32)
+    if fp16v:
+        v = rng.standard_normal((1, 1, n, d)).astype(np.float16)
+        vdev = _lib.v_tiles_f16_swizzled(torch.from_numpy(v).cuda())
+        vor, vs = v.astype(np.float32), None
+    else:
+        vor = rng.integers(0, 120, size=(1, 1, n, d)).astype(np.uint8)
+        vs = np.ones((1, 1, d), np.float32)
+        vdev = _lib.v8_natural_to_tiles(torch.from_numpy(vor).cuda())
+    dev = lambda a: torch.from_numpy(a).cuda()
+    counts = {}
+    for mode in (_lib.PV_PER_BLOCK, _lib.PV_PER_WARP, _lib.PV_NONE):
+        ref, _, refc = oat.block_sparse_attention(q8, k8, vor, lut, valid, thr, qs, ks, vs, d ** -0.5, "fp16",
+                                                  return_pv_count=True, pv="f16" if fp16v else "fp8", pv_mode=mode)
+        out = torch.zeros((1, 1, n, d), dtype=torch.float16, device="cuda")
+        if fp16v:
+            pvc = _lib.block_sparse_attn_f16v(dev(q8), dev(k8), vdev, out, dev(lut), dev(valid), dev(thr), dev(qs), dev(ks),
+                                              d ** -0.5, return_pv_count=True, pv_mode=mode)
+        else:
+            pvc = _lib.block_sparse_attn(dev(q8), dev(k8), vdev, out, dev(lut), dev(valid), dev(thr), dev(qs), dev(ks), dev(vs),
+                                         d ** -0.5, return_pv_count=True, pv_mode=mode)
+        _check_out(out, ref)
+        want = (refc if mode == _lib.PV_PER_WARP else np.repeat(refc[..., None], 4, axis=-1)).reshape(1, 1, 4 * nqb)
+        assert np.array_equal(pvc.cpu().numpy(), want), (mode, pvc, want)
+        counts[mode] = pvc.cpu().numpy().ravel().tolist()
+    assert counts[_lib.PV_PER_BLOCK] == [nblk] * 4 * nqb == counts[_lib.PV_NONE]
+    assert counts[_lib.PV_PER_WARP][1] < nblk and counts[_lib.PV_PER_WARP][:1] + counts[_lib.PV_PER_WARP][2:] == [nblk] * (4 * nqb - 1)

@@ -198,3 +198,46 @@ def test_gqa_equals_mha_with_repeated_kv_heads():
     assert res["k8"].shape[1] == Hkv and rep["k8"].shape[1] == H
     assert np.array_equal(res["out"], rep["out"]) and np.array_equal(res["pv_count"], rep["pv_count"])
     assert not np.array_equal(res["out"][:, 0], res["out"][:, 2])       # heads of different groups do differ
+
+
+def _skip_problem(seed, d=64, nblk=6):
+    """int8 tensors in which block 0 dominates for SOME 32-row groups only, so that the warps of a Q block decide differently."""
+    rng = np.random.default_rng(seed)
+    n = 64 * nblk
+    q8 = rng.integers(-20, 21, size=(1, 1, 128, d)).astype(np.int8)
+    k8 = rng.integers(-20, 21, size=(1, 1, n, d)).astype(np.int8)
+    q8[0, 0, 32:64, 0] = 120                       # rows of group 1 ...
+    k8[0, 0, :64, 0] = 120                         # ... see a huge score on every key of block 0
+    v8 = rng.integers(0, 120, size=(1, 1, n, d)).astype(np.uint8)
+    lut = np.ones((1, 1, 1, nblk), np.int32); lut[0, 0, 0, 0] = 0
+    valid = np.full((1, 1, 1), nblk, np.int32)
+    one = np.ones((1, 1, 1), np.float32)
+    args = dict(pvthreshd=np.array([2.0], np.float32), q_scale=one * 0.05, k_scale=np.full((1, 1, nblk), 0.05, np.float32),
+                v_scale=np.ones((1, 1, d), np.float32), sm_scale=d ** -0.5, out_dtype="fp16")
+    return q8, k8, v8, lut, valid, args
+
+
+def _run(q8, k8, v8, lut, valid, args, **kw):
+    return at.block_sparse_attention(q8, k8, v8, lut, valid, args["pvthreshd"], args["q_scale"], args["k_scale"],
+                                     args["v_scale"], args["sm_scale"], args["out_dtype"], return_pv_count=True, **kw)
+
+
+def test_pv_threshold_modes():
+    q8, k8, v8, lut, valid, args = _skip_problem(5)
+    out1, _, c1 = _run(q8, k8, v8, lut, valid, args, pv_mode=1)
+    out2, _, c2 = _run(q8, k8, v8, lut, valid, args, pv_mode=2)
+    out0, _, c0 = _run(q8, k8, v8, lut, valid, args, pv_mode=0)
+    assert c0[0, 0, 0] == 6 and c1[0, 0, 0] == 6            # the other groups keep the block decision at "compute"
+    assert c2.shape == (1, 1, 1, 4) and c2[0, 0, 0, 1] == 3 and (c2[0, 0, 0, [0, 2, 3]] == 6).all()
+    # never skipping = per-block with a threshold nothing can miss
+    big = dict(args, pvthreshd=np.array([1e6], np.float32))
+    outb, _, _ = _run(q8, k8, v8, lut, valid, big, pv_mode=1)
+    assert np.array_equal(out0, outb)
+    # the per-warp decision of group g is the per-block decision of a Q block made of four copies of group g
+    for g in range(4):
+        qg = np.tile(q8[:, :, 32 * g:32 * g + 32], (1, 1, 4, 1))
+        outg, _, cg = _run(qg, k8, v8, lut, valid, args, pv_mode=1)
+        assert np.array_equal(outg[0, 0, :32], out2[0, 0, 32 * g:32 * g + 32]) and cg[0, 0, 0] == c2[0, 0, 0, g]
+    # skipping changed something for group 1 only
+    assert not np.array_equal(out2[0, 0, 32:64], out1[0, 0, 32:64])
+    assert np.array_equal(out2[0, 0, :32], out1[0, 0, :32]) and np.array_equal(out2[0, 0, 64:], out1[0, 0, 64:])
