@@ -35,6 +35,8 @@ typedef float v16f __attribute__((ext_vector_type(16)));
 
 #define SPG_NEG_BIG (-5000000.0f)   // csrc/qattn/attn_utils.cuh:350, qk_int_sv_f8_cuda_sm89.cuh:171
 #define SPG_FP8_OFFSET 8.807f       // csrc/qattn/attn_utils.cuh:28
+#define SPG_ACC_BIAS_BITS 0x4B400000 // 1.5 * 2^23 as an int32 and ...
+#define SPG_ACC_BIAS 12582912.0f     // ... as a float: floats in [2^23, 2^24) are the integers, one per bit pattern
 #define SPG_LOG2E 1.44269504088896340736f
 
 struct AttnParams {
@@ -67,13 +69,19 @@ __device__ __forceinline__ void lds_wait4(v4i &a, v4i &b, v4i &c, v4i &d) {
   asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(a), "+v"(b), "+v"(c), "+v"(d));
 }
 __device__ __forceinline__ void lds_wait2(v4i &a, v4i &b) { asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(a), "+v"(b)); }
+__device__ __forceinline__ void lds_wait_acc(v16i &a, v16i &b) { asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(a), "+v"(b)); }
 
 // 16-byte-chunk swizzles.  K tile row = key (D bytes, D/16 chunks); V^T tile row = channel (64 bytes, 4 chunks).
-// The functions are chosen such that any 8 consecutive lanes of a ds_read_b128 hit 8 different 16-byte bank groups.
+// The LDS serves a ds_read_b128 one half-wavefront (32 lanes) at a time and needs two clocks for it when the 32
+// addresses fall evenly on the sixteen 16-byte slots of a 256-byte line (two lanes per slot); a slot that is hit 2k
+// times costs k times as much.  The slot of an address is (byte offset mod 256) / 16, so the low row bits already select
+// part of it (one bit for 128-byte rows, two bits for 64-byte rows) and the swizzle must come from OTHER row bits that
+// vary inside a half-wavefront: for the K operand lane r reads key row 32*((r>>2)&1) + 4*(r>>3) + (r&3) (+16 for the
+// second tile), for the V^T operand lane r reads channel row r (+32 per output tile).
 template <int D>
 __device__ __forceinline__ uint32_t k_swz(uint32_t row) {
-  if constexpr (D == 128) return (row & 3u) | (((row >> 5) & 1u) << 2);
-  else return ((row >> 1) & 1u) | (((row >> 5) & 1u) << 1);
+  if constexpr (D == 128) return ((row >> 1) & 3u) | (((row >> 5) & 1u) << 2);
+  else return ((row >> 2) & 1u) | (((row >> 5) & 1u) << 1);
 }
 __device__ __forceinline__ int v_swz(int row) { return (row >> 1) & 3; }
 
@@ -97,10 +105,12 @@ __global__ __launch_bounds__(256, PV16 ? 2 : 3) void block_sparse_attn_kernel(co
   // LDS: K ring [NBUF][TILE] | V^T ring [NBUF][TILE] | votes
   __shared__ __align__(1024) unsigned char smem[NBUF * (TILE + VTILE)];
   __shared__ int sVote[2][4];
+  __shared__ __align__(16) int sBias[4];
   unsigned char *const sKr = smem;
   unsigned char *const sVr = smem + NBUF * TILE;
   const uint32_t lds_k0 = (uint32_t)(size_t)(__attribute__((address_space(3))) unsigned char *)smem;   // LDS byte address
   const uint32_t lds_v0 = lds_k0 + NBUF * TILE;
+  const uint32_t lds_bias = (uint32_t)(size_t)(__attribute__((address_space(3))) int *)sBias;
 
   // ---- workgroup -> (batch*head, q block): one XCD per head at a time, heavy (late) rows first ----------
   const int w = blockIdx.x;
@@ -119,6 +129,7 @@ __global__ __launch_bounds__(256, PV16 ? 2 : 3) void block_sparse_attn_kernel(co
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);   // uniform: everything derived from it stays scalar
   const int N = p.N;
   const int q_row = qb * 128 + wave * 32 + r;
+  if (tid < 4) sBias[tid] = SPG_ACC_BIAS_BITS;   // visible after the barrier that precedes the loop
 
   // ---- Q fragment: B operand of S^T = K.Q^T, resident for the whole loop -------------------------------
   v4i qreg[KS];
@@ -223,6 +234,23 @@ __global__ __launch_bounds__(256, PV16 ? 2 : 3) void block_sparse_attn_kernel(co
   if (nv > 1) SPG_LOAD_TILES(blk1, TILE);
   uint32_t bufoff = 0;                     // LDS ring offset of block it
 
+  // The accumulators start at the bit pattern of 1.5 * 2^23: with |dot| < 2^22 the sums stay inside one binade, so the
+  // int32 result read as a float is exactly 12582912 + dot and no int-to-float conversion is needed.  The pattern is
+  // fetched from LDS (one 16-byte broadcast read per four registers), which costs no vector-ALU slot.  Every read issued
+  // from inline asm is waited for inside the iteration that issued it: the compiler does not know that the destination
+  // registers are written later, so a read still in flight when the loop exits would land on registers it has reused.
+  v16i S0, S1;
+#define SPG_LOAD_BIAS()                                                                                                 \
+  {                                                                                                                     \
+    v4i t0, t1, t2, t3, u0, u1, u2, u3;                                                                                 \
+    asm volatile("ds_read_b128 %0, %8\n\tds_read_b128 %1, %8\n\tds_read_b128 %2, %8\n\tds_read_b128 %3, %8\n\t"        \
+                 "ds_read_b128 %4, %8\n\tds_read_b128 %5, %8\n\tds_read_b128 %6, %8\n\tds_read_b128 %7, %8"               \
+                 : "=&v"(t0), "=&v"(t1), "=&v"(t2), "=&v"(t3), "=&v"(u0), "=&v"(u1), "=&v"(u2), "=&v"(u3)               \
+                 : "v"(lds_bias)                                                                                        \
+                 : "memory");                                                                                           \
+    S0 = (v16i){t0[0], t0[1], t0[2], t0[3], t1[0], t1[1], t1[2], t1[3], t2[0], t2[1], t2[2], t2[3], t3[0], t3[1], t3[2], t3[3]}; \
+    S1 = (v16i){u0[0], u0[1], u0[2], u0[3], u1[0], u1[1], u1[2], u1[3], u2[0], u2[1], u2[2], u2[3], u3[0], u3[1], u3[2], u3[3]}; \
+  }
   __builtin_amdgcn_s_waitcnt(0x0F70);     // vmcnt(0): Q fragment and the first tiles have arrived
   __syncthreads();
 #pragma unroll 1
@@ -232,9 +260,7 @@ __global__ __launch_bounds__(256, PV16 ? 2 : 3) void block_sparse_attn_kernel(co
     const int d4 = it + 4 < nv ? lutc[it + 4] : 0;
 
     // ---- S^T = K . Q^T ---------------------------------------------------------------------------------
-    v16i S0, S1;
-#pragma unroll
-    for (int e = 0; e < 16; e++) { S0[e] = 0; S1[e] = 0; }
+    SPG_LOAD_BIAS();
     {
       // two groups of k-steps: the reads of the second group are in flight while the first group's MFMAs run
       constexpr int HK = KS / 2;
@@ -243,6 +269,7 @@ __global__ __launch_bounds__(256, PV16 ? 2 : 3) void block_sparse_attn_kernel(co
 #pragma unroll
       for (int ks = 0; ks < HK; ks++) lds_read_2x128<0, 16 * D>(a0[ks], a1[ks], kaddr + ((uint32_t)(32 * ks) ^ k_rd_x));
       if constexpr (HK == 2) lds_wait4(a0[0], a1[0], a0[1], a1[1]); else lds_wait2(a0[0], a1[0]);
+      lds_wait_acc(S0, S1);   // the accumulator pattern has arrived as well (same counter); ties S0/S1 to the wait
 #pragma unroll
       for (int ks = HK; ks < KS; ks++) lds_read_2x128<0, 16 * D>(a0[ks], a1[ks], kaddr + ((uint32_t)(32 * ks) ^ k_rd_x));
 #pragma unroll
@@ -260,33 +287,33 @@ __global__ __launch_bounds__(256, PV16 ? 2 : 3) void block_sparse_attn_kernel(co
 
     const float dq = qs * ksc;
     const bool tail = it >= nv - 2;   // last two blocks: masks, no PV skip (sm89.cuh:467-648)
-    float x[32];
-    float a, fm;
+    // S0/S1 are never rewritten (no copies at the join of the two paths): slot e < 16 is S0[e], slot e >= 16 is S1[e - 16]
+    const float a = c * dq;
+    float fm;
+    auto tail_limit = [&]() {
+      const int key0 = blk * 64 + 32 * hh;
+      int lim = 0x7fffffff;
+      if (p.is_causal) lim = q_row - key0;                       // key > query (attn_utils.cuh:334-361)
+      if (it == nv - 1) lim = min(lim, N - 1 - key0);            // key >= kv_len (attn_utils.cuh:363-389)
+      return lim;
+    };
     if (!tail) {
       int imax = S0[0];
 #pragma unroll
       for (int e = 1; e < 16; e++) imax = max(imax, S0[e]);
 #pragma unroll
       for (int e = 0; e < 16; e++) imax = max(imax, S1[e]);
-#pragma unroll
-      for (int e = 0; e < 16; e++) { x[e] = (float)S0[e]; x[16 + e] = (float)S1[e]; }
-      a = c * dq;
-      fm = (float)imax * a;
+      fm = (float)(imax - SPG_ACC_BIAS_BITS) * a;
     } else {
       // slot e of this lane is key 64*blk + 32*hh + e; keys beyond `lim` are masked
-      const int key0 = blk * 64 + 32 * hh;
-      int lim = 0x7fffffff;
-      if (p.is_causal) lim = q_row - key0;                       // key > query (attn_utils.cuh:334-361)
-      if (it == nv - 1) lim = min(lim, N - 1 - key0);            // key >= kv_len (attn_utils.cuh:363-389)
+      const int lim = tail_limit();
       fm = SPG_NEG_BIG;
 #pragma unroll
       for (int e = 0; e < 32; e++) {
-        float v = (float)(e < 16 ? S0[e] : S1[e - 16]) * dq;
+        float v = (__builtin_bit_cast(float, e < 16 ? S0[e] : S1[e - 16]) - SPG_ACC_BIAS) * dq;
         v = e > lim ? SPG_NEG_BIG : v;
-        x[e] = v;
         fm = fmaxf(fm, v);
       }
-      a = c;
       fm = fm * c;
     }
     fm = half_swap_max_f32(fm);
@@ -320,12 +347,25 @@ __global__ __launch_bounds__(256, PV16 ? 2 : 3) void block_sparse_attn_kernel(co
     }
     if (compute) {
       cnt++;
-      const float neg = PV16 ? -m : -m + SPG_FP8_OFFSET;
+      const float neg0 = PV16 ? -m : -m + SPG_FP8_OFFSET;
+      const float neg = __builtin_fmaf(-SPG_ACC_BIAS, a, neg0);   // takes the accumulator bias out: one rounding per row
       float ps = 0.f;
+      float x[32];
+      if (!tail) {
 #pragma unroll
-      for (int e = 0; e < 32; e++) {
-        x[e] = __builtin_amdgcn_exp2f(__builtin_fmaf(x[e], a, neg));
-        if constexpr (!PV16) ps += x[e];
+        for (int e = 0; e < 32; e++) {
+          x[e] = __builtin_amdgcn_exp2f(__builtin_fmaf(__builtin_bit_cast(float, e < 16 ? S0[e] : S1[e - 16]), a, neg));
+          if constexpr (!PV16) ps += x[e];
+        }
+      } else {
+        const int lim = tail_limit();
+        const float masked = __builtin_fmaf(SPG_NEG_BIG, c, neg0);   // what the sentinel score turns into
+#pragma unroll
+        for (int e = 0; e < 32; e++) {
+          const float t = __builtin_fmaf(__builtin_bit_cast(float, e < 16 ? S0[e] : S1[e - 16]), a, neg);
+          x[e] = __builtin_amdgcn_exp2f(e > lim ? masked : t);
+          if constexpr (!PV16) ps += x[e];
+        }
       }
       if constexpr (PV16) {
         typedef _Float16 h8 __attribute__((ext_vector_type(8)));
@@ -428,6 +468,7 @@ __global__ __launch_bounds__(256, PV16 ? 2 : 3) void block_sparse_attn_kernel(co
     bufoff = bufoff == 2 * TILE ? 0 : bufoff + TILE;
   }
 #undef SPG_LOAD_TILES
+#undef SPG_LOAD_BIAS
 #undef SPG_LANE_OFFSETS
 
   // one count per wavefront of 32 query rows, the layout of the reference's PV_Count (sm89.cuh:650-659); the four
