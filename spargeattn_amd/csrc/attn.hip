@@ -352,10 +352,17 @@ __global__ __launch_bounds__(256, PV16 ? 2 : 3) void block_sparse_attn_kernel(co
       float ps = 0.f;
       float x[32];
       if (!tail) {
+        // three passes kept apart for the scheduler: a multiply-add feeding the exponential of the same element directly,
+        // and the exponential feeding the running sum, would issue as one long chain of dependent instructions
 #pragma unroll
-        for (int e = 0; e < 32; e++) {
-          x[e] = __builtin_amdgcn_exp2f(__builtin_fmaf(__builtin_bit_cast(float, e < 16 ? S0[e] : S1[e - 16]), a, neg));
-          if constexpr (!PV16) ps += x[e];
+        for (int e = 0; e < 32; e++) x[e] = __builtin_fmaf(__builtin_bit_cast(float, e < 16 ? S0[e] : S1[e - 16]), a, neg);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int e = 0; e < 32; e++) x[e] = __builtin_amdgcn_exp2f(x[e]);
+        __builtin_amdgcn_sched_barrier(0);
+        if constexpr (!PV16) {
+#pragma unroll
+          for (int e = 0; e < 32; e++) ps += x[e];
         }
       } else {
         const int lim = tail_limit();
