@@ -331,8 +331,11 @@ __global__ __launch_bounds__(256, PV16 ? 2 : 3) void block_sparse_attn_kernel(co
     __syncthreads();   // block it+1's tiles are complete; the votes are visible; ring slot of block it-1 is free
     bool compute = true;
     if (!tail) {       // workgroup-uniform in the per-block mode (sm89.cuh:318-353), wavefront-uniform otherwise
-      const bool any_wave = (sVote[it & 1][0] | sVote[it & 1][1] | sVote[it & 1][2] | sVote[it & 1][3]) != 0;
-      compute = p.pv_mode == 1 ? any_wave : (p.pv_mode == 2 ? vote != 0 : true);
+      compute = p.pv_mode == 0 || vote != 0;
+      // per-block mode: a wavefront whose own vote is set knows the OR already; only one that voted "skip" has to read
+      // what the others wrote (an LDS round trip that the common case does without)
+      if (p.pv_mode == 1 && !compute)
+        compute = (sVote[it & 1][0] | sVote[it & 1][1] | sVote[it & 1][2] | sVote[it & 1][3]) != 0;
     }
     if (it + 2 < nv) {
       const uint32_t b2 = bufoff == 0 ? 2 * TILE : bufoff - TILE;   // slot (it+2) % 3
