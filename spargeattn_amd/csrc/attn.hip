@@ -21,6 +21,9 @@
 //    both the tile hand-over and the workgroup-wide PV-skip vote;
 //  * LDS tiles are unpadded; bank conflicts are avoided by an XOR swizzle of the 16-byte chunks inside a row
 //    (applied to the per-lane global address for K, baked into the HBM tile layout for V);
+//  * the INT8 accumulators start at the bit pattern of 1.5 * 2^23 (read from LDS), so that the int32 result IS the float
+//    12582912 + dot and the scores need no int-to-float conversion; the bias is folded into the constant of the fma
+//    that feeds exp2;
 //  * workgroup ids are remapped so that one XCD (one L2) works on one head at a time, heaviest rows first.
 #include "common.h"
 #include "launch.h"
