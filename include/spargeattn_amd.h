@@ -84,7 +84,7 @@ int spg_map_to_lut(const void *mask, int mask_kind, int32_t *lut, int32_t *valid
  * v (B,H,N,D) dtype (bf16 input is first rounded to fp16, core.py:117).
  * out: v8 e4m3fn codes in TILE layout [B][H][nk][D][64] (key index fastest inside a 64-key tile, rows
  *      beyond N are zero; inside a 64-byte row the four 16-key chunks are XOR-swizzled: key chunk kc is
- *      stored at slot kc ^ ((d >> 1) & 3)) - the layout the attention kernel copies to LDS verbatim;
+ *      stored at slot kc ^ ((d >> 2) & 3)) - the layout the attention kernel copies to LDS verbatim;
  *      v_scale (B,H,D) float32 = amax/2.25.  v_scale doubles as the amax scratch between the passes. */
 int spg_v_quant_fp8(const void *v, uint8_t *v8, float *v_scale, int B, int H, int N, int D, int dtype,
                     void *stream);
@@ -114,7 +114,7 @@ int spg_block_sparse_attn(const int8_t *q8, const int8_t *k8, const uint8_t *v8,
  * with no V scale, is_causal masks at token level.  PV is accumulated in fp32 throughout (the reference rounds each
  * 64-key partial product to fp16 first).
  * spg_v_tiles_f16 prepares the V operand: v (B,H,N,D) fp16|bf16 -> vt (B,H,ceil(N/64),D,64) fp16, the V^T of each
- * 64-key block (bf16 is rounded to fp16 as core.py:247 does), 8-key chunks of a row stored at slot chunk ^ (d & 7),
+ * 64-key block (bf16 is rounded to fp16 as core.py:247 does), 8-key chunks of a row stored at slot chunk ^ ((d >> 1) & 7),
  * zero beyond N.  It takes the place of the kernel's transposing shared-memory reads (ldmatrix.trans). */
 int spg_v_tiles_f16(const void *v, void *vt, int B, int H, int N, int D, int dtype, void *stream);
 int spg_block_sparse_attn_f16v(const int8_t *q8, const int8_t *k8, const void *vt, void *out, int out_dtype,

@@ -168,9 +168,9 @@ def v_quant_fp8(v):
 
 
 def _v_swizzle_index(D, device):
-    """slot index (D,4) such that tile[d, slot] holds key chunk slot ^ ((d >> 1) & 3)."""
+    """slot index (D,4) such that tile[d, slot] holds key chunk slot ^ ((d >> 2) & 3)."""
     d = torch.arange(D, device=device)
-    return torch.arange(4, device=device)[None, :] ^ ((d >> 1) & 3)[:, None]
+    return torch.arange(4, device=device)[None, :] ^ ((d >> 2) & 3)[:, None]
 
 
 def v8_tiles_to_natural(v8):
@@ -220,7 +220,7 @@ def v_tiles_f16_to_natural(vt):
     """(B,H,nk,D,64) swizzled fp16 tiles -> (B,H,nk*64,D) in natural key order."""
     B, H, nk, D, _ = vt.shape
     d = torch.arange(D, device=vt.device)
-    idx = torch.arange(8, device=vt.device)[None, :] ^ (d & 7)[:, None]      # chunk kc sits at slot kc ^ (d & 7)
+    idx = torch.arange(8, device=vt.device)[None, :] ^ ((d >> 1) & 7)[:, None]      # chunk kc sits at slot kc ^ ((d >> 1) & 7)
     t = vt.view(B, H, nk, D, 8, 8)
     nat = torch.gather(t, 4, idx.view(1, 1, 1, D, 8, 1).expand(B, H, nk, D, 8, 8))
     return nat.reshape(B, H, nk, D, 64).permute(0, 1, 2, 4, 3).reshape(B, H, nk * 64, D)

@@ -86,11 +86,11 @@ __device__ __forceinline__ uint32_t k_swz(uint32_t row) {
   if constexpr (D == 128) return ((row >> 1) & 3u) | (((row >> 5) & 1u) << 2);
   else return ((row >> 2) & 1u) | (((row >> 5) & 1u) << 1);
 }
-__device__ __forceinline__ int v_swz(int row) { return (row >> 1) & 3; }
+__device__ __forceinline__ int v_swz(int row) { return (row >> 2) & 3; }
 
 // PV16 = false: V^T tiles are e4m3 (64 bytes per channel row), P is packed to e4m3 with the +8.807 exponent offset and
 //               the denominator sums the un-rounded P (the SageAttention2 kernel, sm89.cuh).
-// PV16 = true:  V^T tiles are fp16 (128 bytes per channel row, 16-byte chunks swizzled by slot = chunk ^ (d & 7)), P is
+// PV16 = true:  V^T tiles are fp16 (128 bytes per channel row, 16-byte chunks swizzled by slot = chunk ^ ((d >> 1) & 7)), P is
 //               rounded to fp16 and the denominator sums the ROUNDED P (the SageAttention1 kernel with the row sum on
 //               the matrix unit, qk_int_sv_f16_cuda_sm80.cuh:339-368, attn_utils.cuh:599-626).  The PV product is
 //               accumulated in fp32; the reference accumulates each 64-key block in fp16 before adding it to its fp32
@@ -212,8 +212,8 @@ __global__ __launch_bounds__(256, PV16 ? 2 : 3) void block_sparse_attn_kernel(co
   const int vsw = v_swz(r);                // v_swz(32*dt + r) does not depend on dt
   // V^T operand: key chunks 2hh and 2hh+1 of channel row r (+32*dt); the two swizzled slots differ in bit 4 only
   const uint32_t v_rd_lo = (uint32_t)(r * 64 + (((2 * hh) ^ vsw) * 16));
-  // fp16 V^T operand of key step s: chunk (4hh + s) ^ (r & 7) of the 128-byte row r (+32*dt): v_rd16 ^ (16 * s)
-  const uint32_t v_rd16 = (uint32_t)(r * 128 + (((4 * hh) ^ (r & 7)) * 16));
+  // fp16 V^T operand of key step s: chunk (4hh + s) ^ ((r >> 1) & 7) of the 128-byte row r (+32*dt): v_rd16 ^ (16 * s)
+  const uint32_t v_rd16 = (uint32_t)(r * 128 + (((4 * hh) ^ ((r >> 1) & 7)) * 16));
 
   float m = SPG_NEG_BIG;
   // d = 1.0 initially (sm89.cuh:172).  FP8 path: each half-lane sums its own 32 keys, so only one of the two starts at 1;

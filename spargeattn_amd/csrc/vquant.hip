@@ -1,6 +1,6 @@
 // V path for gfx950: fp16 cast, per-(b,h,channel) absmax, FP8 e4m3 quantisation written straight into the
 // [B][H][nk][D][64] tile layout the attention kernel's V^T operand reads.  Inside a 64-byte tile row (one channel,
-// 64 keys) the four 16-key chunks are stored XOR-swizzled: key chunk kc sits at slot kc ^ ((d >> 1) & 3), which is
+// 64 keys) the four 16-key chunks are stored XOR-swizzled: key chunk kc sits at slot kc ^ ((d >> 2) & 3), which is
 // the LDS bank-conflict swizzle of the attention kernel baked into the HBM layout (a tile is copied to LDS verbatim).
 // Replaces TransposePadPermuteKernel + MeanScaleKernel (csrc/fused/fused.cu:26-77, 80-191) called with
 // scale_max = 2.25 (spas_sage_attn/core.py:147-151).  HBM-bound: V is read twice (absmax, quantise), written once
@@ -96,14 +96,14 @@ __global__ __launch_bounds__(256) void v_quant_kernel(const uint16_t *__restrict
   uint8_t *out = v8 + ((size_t)bh * nk + blk) * (size_t)(D * 64);
   for (int i = tid; i < D * 4; i += 256) {   // 16-byte pieces: D rows x 4 slots
     const int d = i >> 2, slot = i & 3;
-    const int kc = slot ^ ((d >> 1) & 3);      // key chunk stored in this slot
+    const int kc = slot ^ ((d >> 2) & 3);      // key chunk stored in this slot
     const uint32_t *src = (const uint32_t *)(tile + d * LDW + kc * 16);
     *(uint4 *)(out + d * 64 + slot * 16) = make_uint4(src[0], src[1], src[2], src[3]);
   }
 }
 
 // V -> fp16 -> V^T tiles [nk][D][64] fp16 for the fp16-PV attention variant.  Inside a 128-byte tile row (one channel,
-// 64 keys) the eight 8-key chunks are stored at slot = chunk ^ (d & 7) (the LDS swizzle of the attention kernel).
+// 64 keys) the eight 8-key chunks are stored at slot = chunk ^ ((d >> 1) & 7) (the LDS swizzle of the attention kernel).
 // Keys at or beyond N are zero.  One workgroup per 64-key tile.
 template <int D, int DT>
 __global__ __launch_bounds__(256) void v_tiles_f16_kernel(const uint16_t *__restrict__ v, uint16_t *__restrict__ vt,
@@ -137,7 +137,7 @@ __global__ __launch_bounds__(256) void v_tiles_f16_kernel(const uint16_t *__rest
   uint16_t *out = vt + ((size_t)bh * nk + blk) * (size_t)(D * 64);
   for (int i = tid; i < D * 8; i += 256) {   // 16-byte pieces: D rows x 8 slots
     const int d = i >> 3, slot = i & 7;
-    const int kc = slot ^ (d & 7);             // key chunk stored in this slot
+    const int kc = slot ^ ((d >> 1) & 7);      // key chunk stored in this slot
     const uint16_t *src = tile + d * LDW + kc * 8;
     uint32_t o[4];
 #pragma unroll
