@@ -47,20 +47,30 @@ enum spg_mask_kind {
 int spg_version(void);
 const char *spg_last_error(void);
 
+/* Strides.  The tensors the CALLER owns in its own layout - q, k, v going in, the attention output coming out - are
+ * described by a pointer plus `const int64_t *strides`: NULL for a contiguous (B,H,N,D) tensor ("HND"), or a HOST array
+ * {batch, head, row} of element strides with the last dimension contiguous, e.g. {N*H*D, D, H*D} for a contiguous
+ * (B,N,H,D) tensor ("NHD").  This is what tensor_layout and the stride arguments of the reference's kernels carry
+ * (csrc/qattn/qk_int_sv_f8_cuda_sm89.cu:256-300; the Python API copies NHD inputs to HND first, core.py:109-117, which
+ * a caller of this library need not do).  Rows move in 16-byte pieces: every stride is a positive multiple of 8
+ * elements and the pointer is 16-byte aligned.  Everything the library produces for itself (int8 tensors, scales,
+ * pooled blocks, LUT, FP8 tiles) is contiguous HND. */
+
 /* ---- A2: km = k.mean(dim=-2)  (spas_sage_attn/core.py:119-120) -------------------------------
- * k (B,H,N,D) dtype -> km (B,H,D) dtype.  Column sums are accumulated in binary64 and rounded once.
+ * k (B,H,N,D) dtype, strided -> km (B,H,D) dtype.  Column sums are accumulated in binary64 and rounded once.
  * workspace: spg_km_mean_workspace_bytes() bytes of device scratch (per-chunk partial sums). */
 size_t spg_km_mean_workspace_bytes(int B, int H, int N, int D);
-int spg_km_mean(const void *k, void *km, void *workspace, int B, int H, int N, int D, int dtype, void *stream);
+int spg_km_mean(const void *k, const int64_t *k_strides, void *km, void *workspace, int B, int H, int N, int D, int dtype,
+                void *stream);
 
 /* ---- A3/A4: fused pool + self-similarity + per-block INT8 quantisation ------------------------
  * replaces triton_bmm_pool_sim_simmean_fuse_quant (spas_sage_attn/utils.py:161-214, wrapper 270-280).
- * x (B,H,N,D) dtype; km (B,H,D) dtype or NULL (Q: NULL, K: the column mean, subtracted in dtype);
+ * x (B,H,N,D) dtype, strided; km (B,H,D) dtype or NULL (Q: NULL, K: the column mean, subtracted in dtype);
  * block = 128 (Q) or 64 (K); simthreshd1 (H,) float32.
  * out: pool (B,H,nb,D) dtype; sim (B,H,nb) uint8 0/1; xq (B,H,N,D) int8; scale (B,H,nb) float32.
  * ---- A13: with pool == NULL and sim == NULL this is qk_quantize (utils.py:89-159): xq and scale only. */
-int spg_pool_sim_quant(const void *x, const void *km, void *pool, uint8_t *sim, int8_t *xq, float *scale,
-                       const float *simthreshd1, int B, int H, int N, int D, int block, int dtype, void *stream);
+int spg_pool_sim_quant(const void *x, const int64_t *x_strides, const void *km, void *pool, uint8_t *sim, int8_t *xq,
+                       float *scale, const float *simthreshd1, int B, int H, int N, int D, int block, int dtype, void *stream);
 
 /* ---- A5-A8: compressed attention, top-k / CDF selection, block map, LUT ------------------------
  * replaces the torch glue of get_block_map_meansim_fuse_quant (spas_sage_attn/utils.py:386-420),
@@ -81,28 +91,28 @@ int spg_map_to_lut(const void *mask, int mask_kind, int32_t *lut, int32_t *valid
 /* ---- A9+A10: V -> fp16 -> per-channel FP8 e4m3 ---------------------------------------------------
  * replaces transpose_pad_permute_cuda + scale_fuse_quant_cuda(..., scale_max = 2.25)
  * (csrc/fused/fused.cu:193-267, 269-344; called at core.py:147,151).
- * v (B,H,N,D) dtype (bf16 input is first rounded to fp16, core.py:117).
+ * v (B,H,N,D) dtype, strided (bf16 input is first rounded to fp16, core.py:117).
  * out: v8 e4m3fn codes in TILE layout [B][H][nk][D][64] (key index fastest inside a 64-key tile, rows
  *      beyond N are zero; inside a 64-byte row the four 16-key chunks are XOR-swizzled: key chunk kc is
  *      stored at slot kc ^ ((d >> 2) & 3)) - the layout the attention kernel copies to LDS verbatim;
  *      v_scale (B,H,D) float32 = amax/2.25.  v_scale doubles as the amax scratch between the passes. */
-int spg_v_quant_fp8(const void *v, uint8_t *v8, float *v_scale, int B, int H, int N, int D, int dtype,
-                    void *stream);
+int spg_v_quant_fp8(const void *v, const int64_t *v_strides, uint8_t *v8, float *v_scale, int B, int H, int N, int D,
+                    int dtype, void *stream);
 
 /* ---- A11: block-sparse INT8-QK / FP8-PV attention ------------------------------------------------
  * replaces qk_int8_sv_f8_accum_f32_block_sparse_attn_inst_buf_fuse_v_scale_with_pv_threshold
  * (csrc/qattn/attn_cuda.h:61-76, csrc/qattn/qk_int_sv_f8_cuda_sm89.cu:197-390) with
  * tensor_layout = HND, qk_quant_gran = per-block; pv_threshold_mode = SPG_PV_PER_BLOCK is what that entry point
  * compiles in (sm89.cu:365), the other two modes are the kernel template's (sm89.cuh:283-391).
- * q8 int8 (B,H,N,D); k8 int8 (B,Hkv,N,D); v8 as produced by spg_v_quant_fp8 for Hkv heads; out (B,H,N,D) out_dtype;
+ * q8 int8 (B,H,N,D); k8 int8 (B,Hkv,N,D); v8 as produced by spg_v_quant_fp8 for Hkv heads; out (B,H,N,D) out_dtype, strided;
  * lut/valid_block_num as above; pvthreshd (H,) float32; q_scale (B,H,nq), k_scale (B,Hkv,nk),
  * v_scale (B,Hkv,D) float32; Hkv divides H: query head h reads K/V head h / (H / Hkv) (grouped-query attention,
  * sm89.cu:310-314, sm89.cuh:118); Hkv = H is plain multi-head attention; pv_count (B,H,nq*4) int32 or NULL: number of K blocks
  * whose PV was computed, one entry per 32 query rows as in the reference (sm89.cu:331-334); entries of Q blocks with
  * valid_block_num == 0 are left untouched.
  * Row blocks with valid_block_num == 0 are left unwritten, as in the reference (sm89.cuh:232-235). */
-int spg_block_sparse_attn(const int8_t *q8, const int8_t *k8, const uint8_t *v8, void *out, int out_dtype,
-                          const int32_t *lut, const int32_t *valid_block_num, const float *pvthreshd,
+int spg_block_sparse_attn(const int8_t *q8, const int8_t *k8, const uint8_t *v8, void *out, const int64_t *out_strides,
+                          int out_dtype, const int32_t *lut, const int32_t *valid_block_num, const float *pvthreshd,
                           const float *q_scale, const float *k_scale, const float *v_scale,
                           int B, int H, int Hkv, int N, int D, float sm_scale, int is_causal, int pv_threshold_mode,
                           int32_t *pv_count, void *stream);
@@ -116,9 +126,9 @@ int spg_block_sparse_attn(const int8_t *q8, const int8_t *k8, const uint8_t *v8,
  * spg_v_tiles_f16 prepares the V operand: v (B,H,N,D) fp16|bf16 -> vt (B,H,ceil(N/64),D,64) fp16, the V^T of each
  * 64-key block (bf16 is rounded to fp16 as core.py:247 does), 8-key chunks of a row stored at slot chunk ^ ((d >> 1) & 7),
  * zero beyond N.  It takes the place of the kernel's transposing shared-memory reads (ldmatrix.trans). */
-int spg_v_tiles_f16(const void *v, void *vt, int B, int H, int N, int D, int dtype, void *stream);
-int spg_block_sparse_attn_f16v(const int8_t *q8, const int8_t *k8, const void *vt, void *out, int out_dtype,
-                               const int32_t *lut, const int32_t *valid_block_num, const float *pvthreshd,
+int spg_v_tiles_f16(const void *v, const int64_t *v_strides, void *vt, int B, int H, int N, int D, int dtype, void *stream);
+int spg_block_sparse_attn_f16v(const int8_t *q8, const int8_t *k8, const void *vt, void *out, const int64_t *out_strides,
+                               int out_dtype, const int32_t *lut, const int32_t *valid_block_num, const float *pvthreshd,
                                const float *q_scale, const float *k_scale,
                                int B, int H, int Hkv, int N, int D, float sm_scale, int is_causal, int pv_threshold_mode,
                                int32_t *pv_count, void *stream);

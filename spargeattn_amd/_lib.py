@@ -24,14 +24,14 @@ SIGNATURES = {
     "spg_version": (_i, []),
     "spg_last_error": (_c.c_char_p, []),
     "spg_km_mean_workspace_bytes": (_sz, [_i, _i, _i, _i]),
-    "spg_km_mean": (_i, [_vp, _vp, _vp, _i, _i, _i, _i, _i, _vp]),
-    "spg_pool_sim_quant": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp]),
+    "spg_km_mean": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp]),
+    "spg_pool_sim_quant": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp]),
     "spg_block_select": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp]),
     "spg_map_to_lut": (_i, [_vp, _i, _vp, _vp, _i, _i, _i, _i, _vp]),
-    "spg_v_quant_fp8": (_i, [_vp, _vp, _vp, _i, _i, _i, _i, _i, _vp]),
-    "spg_block_sparse_attn": (_i, [_vp, _vp, _vp, _vp, _i, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _f, _i, _i, _vp, _vp]),
-    "spg_v_tiles_f16": (_i, [_vp, _vp, _i, _i, _i, _i, _i, _vp]),
-    "spg_block_sparse_attn_f16v": (_i, [_vp] * 4 + [_i] + [_vp] * 5 + [_i] * 5 + [_f, _i, _i, _vp, _vp]),
+    "spg_v_quant_fp8": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp]),
+    "spg_block_sparse_attn": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _f, _i, _i, _vp, _vp]),
+    "spg_v_tiles_f16": (_i, [_vp, _vp, _vp, _i, _i, _i, _i, _i, _vp]),
+    "spg_block_sparse_attn_f16v": (_i, [_vp] * 5 + [_i] + [_vp] * 5 + [_i] * 5 + [_f, _i, _i, _vp, _vp]),
     "spg_dense_attn_f16": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _f, _i, _vp]),
     "spg_selftest_division": (_i, [_vp, _i, ctypes.c_uint, _vp]),
 }
@@ -90,6 +90,24 @@ def _p(t):
     return None if t is None else t.data_ptr()
 
 
+def _dev_strided(*ts):
+    """GPU tensors (B,H,N,D) whose last dimension is contiguous; the other strides are free (HND, NHD views, slices)."""
+    for t in ts:
+        if not t.is_cuda:
+            raise RuntimeError("spargeattn_amd kernels need GPU tensors (there is no CPU path)")
+        if t.dim() != 4 or t.stride(3) != 1:
+            raise RuntimeError("expected a 4-D tensor whose last dimension is contiguous")
+        if any(st % 8 for st in t.stride()[:3]) or t.data_ptr() % 16:
+            raise RuntimeError("rows must be 16-byte aligned (strides multiples of 8 elements)")
+
+
+def _st(t):
+    """{batch, head, row} element strides as the host array the C ABI takes (NULL when contiguous)."""
+    if t.is_contiguous():
+        return None
+    return (ctypes.c_int64 * 3)(t.stride(0), t.stride(1), t.stride(2))
+
+
 def _stream():
     return torch.cuda.current_stream().cuda_stream
 
@@ -106,18 +124,19 @@ _MASK_KIND = {
 
 def km_mean(k):
     """k (B,H,N,D) -> km (B,H,1,D), same dtype."""
-    _dev(k)
+    _dev_strided(k)
     B, H, N, D = k.shape
     lib = load()
     km = torch.empty((B, H, 1, D), dtype=k.dtype, device=k.device)
     ws = torch.empty(max(1, lib.spg_km_mean_workspace_bytes(B, H, N, D)), dtype=torch.uint8, device=k.device)
-    _check(lib.spg_km_mean(_p(k), _p(km), _p(ws), B, H, N, D, _dt(k), _stream()))
+    _check(lib.spg_km_mean(_p(k), _st(k), _p(km), _p(ws), B, H, N, D, _dt(k), _stream()))
     return km
 
 
 def pool_sim_quant(x, km, block, simthreshd1=None, with_pool=True):
     """Returns (pool, sim, x_int8, scale) - pool and sim are None when with_pool is False."""
-    _dev(x, km, simthreshd1)
+    _dev_strided(x)
+    _dev(km, simthreshd1)
     B, H, N, D = x.shape
     nb = (N + block - 1) // block
     xq = torch.empty((B, H, N, D), dtype=torch.int8, device=x.device)
@@ -126,7 +145,7 @@ def pool_sim_quant(x, km, block, simthreshd1=None, with_pool=True):
     if with_pool:
         pool = torch.empty((B, H, nb, D), dtype=x.dtype, device=x.device)
         sim = torch.empty((B, H, nb), dtype=torch.bool, device=x.device)
-    _check(load().spg_pool_sim_quant(_p(x), _p(km), _p(pool), _p(sim), _p(xq), _p(scale), _p(simthreshd1),
+    _check(load().spg_pool_sim_quant(_p(x), _st(x), _p(km), _p(pool), _p(sim), _p(xq), _p(scale), _p(simthreshd1),
                                      B, H, N, D, block, _dt(x), _stream()))
     return pool, sim, xq, scale
 
@@ -158,12 +177,12 @@ def map_to_lut(block_map):
 
 def v_quant_fp8(v):
     """v (B,H,N,D) fp16/bf16 -> (v8 uint8 codes in tile layout (B,H,nk,D,64), v_scale (B,H,D) float32)."""
-    _dev(v)
+    _dev_strided(v)
     B, H, N, D = v.shape
     nk = (N + 63) // 64
     v8 = torch.empty((B, H, nk, D, 64), dtype=torch.uint8, device=v.device)
     v_scale = torch.empty((B, H, D), dtype=torch.float32, device=v.device)
-    _check(load().spg_v_quant_fp8(_p(v), _p(v8), _p(v_scale), B, H, N, D, _dt(v), _stream()))
+    _check(load().spg_v_quant_fp8(_p(v), _st(v), _p(v8), _p(v_scale), B, H, N, D, _dt(v), _stream()))
     return v8, v_scale
 
 
@@ -197,10 +216,11 @@ PV_NONE, PV_PER_BLOCK, PV_PER_WARP = 0, 1, 2
 
 def block_sparse_attn(q8, k8, v8, out, lut, valid, pvthreshd, q_scale, k_scale, v_scale, sm_scale,
                       is_causal=False, return_pv_count=False, pv_mode=PV_PER_BLOCK):
-    _dev(q8, k8, v8, out, lut, valid, pvthreshd, q_scale, k_scale, v_scale)
+    _dev(q8, k8, v8, lut, valid, pvthreshd, q_scale, k_scale, v_scale)
+    _dev_strided(out)
     B, H, N, D = q8.shape
     pvc = torch.zeros((B, H, 4 * ((N + 127) // 128)), dtype=torch.int32, device=q8.device) if return_pv_count else None
-    _check(load().spg_block_sparse_attn(_p(q8), _p(k8), _p(v8), _p(out), _dt(out), _p(lut), _p(valid), _p(pvthreshd),
+    _check(load().spg_block_sparse_attn(_p(q8), _p(k8), _p(v8), _p(out), _st(out), _dt(out), _p(lut), _p(valid), _p(pvthreshd),
                                         _p(q_scale), _p(k_scale), _p(v_scale), B, H, k8.shape[1], N, D, float(sm_scale),
                                         int(bool(is_causal)), int(pv_mode), _p(pvc), _stream()))
     return pvc
@@ -208,11 +228,11 @@ def block_sparse_attn(q8, k8, v8, out, lut, valid, pvthreshd, q_scale, k_scale, 
 
 def v_tiles_f16_swizzled(v):
     """v (B,H,N,D) fp16/bf16 -> (B,H,nk,D,64) fp16 V^T tiles, chunk-swizzled, the operand of block_sparse_attn_f16v."""
-    _dev(v)
+    _dev_strided(v)
     B, H, N, D = v.shape
     nk = (N + 63) // 64
     vt = torch.empty((B, H, nk, D, 64), dtype=torch.float16, device=v.device)
-    _check(load().spg_v_tiles_f16(_p(v), _p(vt), B, H, N, D, _dt(v), _stream()))
+    _check(load().spg_v_tiles_f16(_p(v), _st(v), _p(vt), B, H, N, D, _dt(v), _stream()))
     return vt
 
 
@@ -228,10 +248,11 @@ def v_tiles_f16_to_natural(vt):
 
 def block_sparse_attn_f16v(q8, k8, vt, out, lut, valid, pvthreshd, q_scale, k_scale, sm_scale, is_causal=False,
                            return_pv_count=False, pv_mode=PV_PER_BLOCK):
-    _dev(q8, k8, vt, out, lut, valid, pvthreshd, q_scale, k_scale)
+    _dev(q8, k8, vt, lut, valid, pvthreshd, q_scale, k_scale)
+    _dev_strided(out)
     B, H, N, D = q8.shape
     pvc = torch.zeros((B, H, 4 * ((N + 127) // 128)), dtype=torch.int32, device=q8.device) if return_pv_count else None
-    _check(load().spg_block_sparse_attn_f16v(_p(q8), _p(k8), _p(vt), _p(out), _dt(out), _p(lut), _p(valid),
+    _check(load().spg_block_sparse_attn_f16v(_p(q8), _p(k8), _p(vt), _p(out), _st(out), _dt(out), _p(lut), _p(valid),
                                              _p(pvthreshd), _p(q_scale), _p(k_scale), B, H, k8.shape[1], N, D, float(sm_scale),
                                              int(bool(is_causal)), int(pv_mode), _p(pvc), _stream()))
     return pvc

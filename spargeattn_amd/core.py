@@ -40,12 +40,35 @@ def _prologue(q, k, v, tensor_layout):
         raise RuntimeError("spargeattn_amd needs GPU tensors (there is no CPU path)")
     torch.cuda.set_device(v.device)
     qk_dtype = torch.bfloat16 if q.dtype == torch.bfloat16 else torch.float16
-    q = q.contiguous().to(qk_dtype)
-    k = k.contiguous().to(qk_dtype)
+    # The reference makes contiguous HND copies here (core.py:113-117).  The kernels that read q, k, v take strides, so
+    # an NHD tensor (or any view whose rows are contiguous and 16-byte aligned) is read where it lies; only other
+    # layouts and dtypes are copied.
+    q = _rows_ok(q).to(qk_dtype)
+    k = _rows_ok(k).to(qk_dtype)
     # V is always quantised from fp16 (core.py:117).  A bf16 V is handed over as it is: the quantisation kernel
     # rounds each element to fp16 in registers, which gives the same values without a pass over HBM.
-    v = v.contiguous() if v.dtype in (torch.float16, torch.bfloat16) else v.contiguous().to(torch.float16)
+    v = _rows_ok(v)
+    if v.dtype not in (torch.float16, torch.bfloat16):
+        v = v.to(torch.float16)
     return q, k, v
+
+
+def _rows_ok(t):
+    """t itself if the strided kernels can read it (last dimension contiguous, 16-byte aligned rows), else a copy."""
+    esz = t.element_size()
+    ok = (t.stride(-1) == 1 and t.data_ptr() % 16 == 0 and t.dtype in (torch.float16, torch.bfloat16)
+          and all((st * esz) % 16 == 0 for st in t.stride()[:-1]))
+    return t if ok else t.contiguous()
+
+
+def _empty_out(q):
+    """Output buffer with q's shape whose MEMORY layout follows q's (an NHD view gets an NHD buffer, so that the
+    transpose back at the end is a view of contiguous memory)."""
+    if q.is_contiguous():
+        return torch.empty_like(q)
+    if q.transpose(-2, -3).is_contiguous():
+        return torch.empty_like(q.transpose(-2, -3)).transpose(-2, -3)
+    return torch.empty(q.shape, dtype=q.dtype, device=q.device)
 
 
 def _attention(q, k, v, q_int8, q_scale, k_int8, k_scale, lut, valid_block_num, scale, pvthreshd, kernel_causal,
@@ -55,7 +78,7 @@ def _attention(q, k, v, q_int8, q_scale, k_int8, k_scale, lut, valid_block_num, 
         scale = 1.0 / (headdim ** 0.5)
     assert headdim in [64, 128], "headdim should be in [64, 128]. For other headdim, you can use padding and specify the softmax scale."
     pvthreshd = hyperparameter_check(pvthreshd, q.size(-3), q.device)
-    o = torch.empty_like(q)
+    o = _empty_out(q)
     _mark("vquant")
     v_fp8, v_scale = _lib.v_quant_fp8(v)
     _mark("attn")
@@ -110,7 +133,7 @@ def _meansim_sage1(q, k, v, is_causal, scale, smooth_k, simthreshd1, cdfthreshd,
         scale = 1.0 / (headdim ** 0.5)
     assert headdim in [64, 128], "headdim should be in [64, 128]. For other headdim, you can use padding and specify the softmax scale."
     pvthreshd = hyperparameter_check(pvthreshd, q.size(-3), q.device)
-    o = torch.empty_like(q)
+    o = _empty_out(q)
     _mark("vquant")
     vt = _lib.v_tiles_f16_swizzled(v)
     _mark("attn")

@@ -46,6 +46,7 @@ struct AttnParams {
   const int8_t *q8, *k8;
   const uint8_t *v8;
   void *out;
+  Strides os;      // element strides of out (B, H, N, D), last dimension contiguous
   const int32_t *lut, *valid;
   const float *pvthr, *q_scale, *k_scale, *v_scale;
   int32_t *pv_count;
@@ -492,7 +493,7 @@ __global__ __launch_bounds__(256, PV16 ? 2 : 3) void block_sparse_attn_kernel(co
   const float dtot = PV16 ? dsum : half_swap_sum_f32(dsum);
   const float inv = __builtin_amdgcn_rcpf(dtot);
   if (q_row < N) {
-    uint16_t *orow = (uint16_t *)p.out + ((size_t)bh * N + q_row) * D;
+    uint16_t *orow = (uint16_t *)p.out + (size_t)(bh / p.H) * p.os.sb + (size_t)head * p.os.sh + (size_t)q_row * p.os.sn;
     const float *vs = p.v_scale + (size_t)bhk * D;
 #pragma unroll
     for (int dt = 0; dt < NDT; dt++) {
@@ -511,13 +512,13 @@ __global__ __launch_bounds__(256, PV16 ? 2 : 3) void block_sparse_attn_kernel(co
   }
 }
 
-hipError_t launch_block_sparse_attn(const int8_t *q8, const int8_t *k8, const uint8_t *v8, void *out, int out_dtype,
-                                    const int32_t *lut, const int32_t *valid, const float *pvthreshd,
+hipError_t launch_block_sparse_attn(const int8_t *q8, const int8_t *k8, const uint8_t *v8, void *out, Strides os,
+                                    int out_dtype, const int32_t *lut, const int32_t *valid, const float *pvthreshd,
                                     const float *q_scale, const float *k_scale, const float *v_scale, int B, int H,
                                     int Hkv, int N, int D, float sm_scale, int is_causal, int pv_mode,
                                     int32_t *pv_count, hipStream_t st) {
   AttnParams p;
-  p.q8 = q8; p.k8 = k8; p.v8 = v8; p.out = out; p.lut = lut; p.valid = valid; p.pvthr = pvthreshd;
+  p.q8 = q8; p.k8 = k8; p.v8 = v8; p.out = out; p.os = os; p.lut = lut; p.valid = valid; p.pvthr = pvthreshd;
   p.q_scale = q_scale; p.k_scale = k_scale; p.v_scale = v_scale; p.pv_count = pv_count;
   p.B = B; p.H = H; p.Hkv = Hkv; p.N = N; p.nq = (N + 127) / 128; p.nk = (N + 63) / 64;
   p.sm_scale_log2 = sm_scale * SPG_LOG2E;

@@ -49,6 +49,21 @@ int check_dtype(const char *fn, int dtype) {
   return SPG_OK;
 }
 
+// strides == NULL: HND-contiguous.  Otherwise {batch, head, row} strides in elements; rows are read and written in
+// 16-byte pieces, so every stride must be a multiple of 8 elements and a row must not overlap the next one.
+int get_strides(const char *fn, const char *what, const int64_t *strides, int H, int N, int D, spg::Strides *out) {
+  if (strides == nullptr) {
+    out->sb = (long long)H * N * D; out->sh = (long long)N * D; out->sn = D;
+    return SPG_OK;
+  }
+  for (int i = 0; i < 3; i++)
+    if (strides[i] <= 0 || strides[i] % 8 != 0)
+      return fail(SPG_ERR_INVALID, "%s: %s[%d] = %lld must be a positive multiple of 8 elements", fn, what, i, (long long)strides[i]);
+  if (strides[2] < D) return fail(SPG_ERR_INVALID, "%s: %s[2] = %lld is smaller than head_dim %d", fn, what, (long long)strides[2], D);
+  out->sb = strides[0]; out->sh = strides[1]; out->sn = strides[2];
+  return SPG_OK;
+}
+
 #define SPG_TRY(expr) do { int rc_ = (expr); if (rc_ != SPG_OK) return rc_; } while (0)
 #define SPG_NONNULL(fn, ptr) do { if ((ptr) == nullptr) return fail(SPG_ERR_INVALID, "%s: %s is NULL", fn, #ptr); } while (0)
 }  // namespace
@@ -64,16 +79,18 @@ size_t spg_km_mean_workspace_bytes(int B, int H, int N, int D) {
   return spg::km_mean_workspace_bytes(B, H, N, D);
 }
 
-int spg_km_mean(const void *k, void *km, void *workspace, int B, int H, int N, int D, int dtype, void *stream) {
+int spg_km_mean(const void *k, const int64_t *k_strides, void *km, void *workspace, int B, int H, int N, int D, int dtype, void *stream) {
   const char *fn = "spg_km_mean";
   SPG_TRY(check_shape(fn, B, H, N, D));
   SPG_TRY(check_dtype(fn, dtype));
   SPG_NONNULL(fn, k); SPG_NONNULL(fn, km); SPG_NONNULL(fn, workspace);
-  spg::launch_km_mean(k, km, workspace, B, H, N, D, dtype, (hipStream_t)stream);
+  spg::Strides ks;
+  SPG_TRY(get_strides(fn, "k_strides", k_strides, H, N, D, &ks));
+  spg::launch_km_mean(k, ks, km, workspace, B, H, N, D, dtype, (hipStream_t)stream);
   return check_launch(fn, hipSuccess);
 }
 
-int spg_pool_sim_quant(const void *x, const void *km, void *pool, uint8_t *sim, int8_t *xq, float *scale,
+int spg_pool_sim_quant(const void *x, const int64_t *x_strides, const void *km, void *pool, uint8_t *sim, int8_t *xq, float *scale,
                        const float *simthreshd1, int B, int H, int N, int D, int block, int dtype, void *stream) {
   const char *fn = "spg_pool_sim_quant";
   SPG_TRY(check_shape(fn, B, H, N, D));
@@ -82,7 +99,9 @@ int spg_pool_sim_quant(const void *x, const void *km, void *pool, uint8_t *sim, 
   SPG_NONNULL(fn, x); SPG_NONNULL(fn, xq); SPG_NONNULL(fn, scale);
   if ((pool == nullptr) != (sim == nullptr)) return fail(SPG_ERR_INVALID, "%s: pool and sim must both be given or both be NULL", fn);
   if (pool != nullptr) SPG_NONNULL(fn, simthreshd1);
-  spg::launch_pool_sim_quant(x, km, pool, sim, xq, scale, simthreshd1, B, H, N, D, block, dtype, (hipStream_t)stream);
+  spg::Strides xs;
+  SPG_TRY(get_strides(fn, "x_strides", x_strides, H, N, D, &xs));
+  spg::launch_pool_sim_quant(x, xs, km, pool, sim, xq, scale, simthreshd1, B, H, N, D, block, dtype, (hipStream_t)stream);
   return check_launch(fn, hipSuccess);
 }
 
@@ -123,16 +142,19 @@ int spg_selftest_division(unsigned long long *counts, int n_divisors, unsigned i
   return check_launch(fn, hipSuccess);
 }
 
-int spg_v_quant_fp8(const void *v, uint8_t *v8, float *v_scale, int B, int H, int N, int D, int dtype, void *stream) {
+int spg_v_quant_fp8(const void *v, const int64_t *v_strides, uint8_t *v8, float *v_scale, int B, int H, int N, int D, int dtype, void *stream) {
   const char *fn = "spg_v_quant_fp8";
   SPG_TRY(check_shape(fn, B, H, N, D));
   SPG_TRY(check_dtype(fn, dtype));
   SPG_NONNULL(fn, v); SPG_NONNULL(fn, v8); SPG_NONNULL(fn, v_scale);
-  spg::launch_v_quant_fp8(v, v8, v_scale, B, H, N, D, dtype, (hipStream_t)stream);
+  spg::Strides vs;
+  SPG_TRY(get_strides(fn, "v_strides", v_strides, H, N, D, &vs));
+  spg::launch_v_quant_fp8(v, vs, v8, v_scale, B, H, N, D, dtype, (hipStream_t)stream);
   return check_launch(fn, hipSuccess);
 }
 
-int spg_block_sparse_attn(const int8_t *q8, const int8_t *k8, const uint8_t *v8, void *out, int out_dtype,
+int spg_block_sparse_attn(const int8_t *q8, const int8_t *k8, const uint8_t *v8, void *out, const int64_t *out_strides,
+                          int out_dtype,
                           const int32_t *lut, const int32_t *valid_block_num, const float *pvthreshd,
                           const float *q_scale, const float *k_scale, const float *v_scale, int B, int H, int Hkv, int N,
                           int D, float sm_scale, int is_causal, int pv_threshold_mode, int32_t *pv_count, void *stream) {
@@ -144,21 +166,26 @@ int spg_block_sparse_attn(const int8_t *q8, const int8_t *k8, const uint8_t *v8,
   SPG_NONNULL(fn, q8); SPG_NONNULL(fn, k8); SPG_NONNULL(fn, v8); SPG_NONNULL(fn, out); SPG_NONNULL(fn, lut);
   SPG_NONNULL(fn, valid_block_num); SPG_NONNULL(fn, pvthreshd); SPG_NONNULL(fn, q_scale); SPG_NONNULL(fn, k_scale);
   SPG_NONNULL(fn, v_scale);
-  return check_launch(fn, spg::launch_block_sparse_attn(q8, k8, v8, out, out_dtype, lut, valid_block_num, pvthreshd,
+  spg::Strides os;
+  SPG_TRY(get_strides(fn, "out_strides", out_strides, H, N, D, &os));
+  return check_launch(fn, spg::launch_block_sparse_attn(q8, k8, v8, out, os, out_dtype, lut, valid_block_num, pvthreshd,
                                                         q_scale, k_scale, v_scale, B, H, Hkv, N, D, sm_scale,
                                                         is_causal ? 1 : 0, pv_threshold_mode, pv_count, (hipStream_t)stream));
 }
 
-int spg_v_tiles_f16(const void *v, void *vt, int B, int H, int N, int D, int dtype, void *stream) {
+int spg_v_tiles_f16(const void *v, const int64_t *v_strides, void *vt, int B, int H, int N, int D, int dtype, void *stream) {
   const char *fn = "spg_v_tiles_f16";
   SPG_TRY(check_shape(fn, B, H, N, D));
   SPG_TRY(check_dtype(fn, dtype));
   SPG_NONNULL(fn, v); SPG_NONNULL(fn, vt);
-  spg::launch_v_tiles_f16(v, vt, B, H, N, D, dtype, (hipStream_t)stream);
+  spg::Strides vs;
+  SPG_TRY(get_strides(fn, "v_strides", v_strides, H, N, D, &vs));
+  spg::launch_v_tiles_f16(v, vs, vt, B, H, N, D, dtype, (hipStream_t)stream);
   return check_launch(fn, hipSuccess);
 }
 
-int spg_block_sparse_attn_f16v(const int8_t *q8, const int8_t *k8, const void *vt, void *out, int out_dtype,
+int spg_block_sparse_attn_f16v(const int8_t *q8, const int8_t *k8, const void *vt, void *out, const int64_t *out_strides,
+                               int out_dtype,
                                const int32_t *lut, const int32_t *valid_block_num, const float *pvthreshd,
                                const float *q_scale, const float *k_scale, int B, int H, int Hkv, int N, int D,
                                float sm_scale, int is_causal, int pv_threshold_mode, int32_t *pv_count, void *stream) {
@@ -169,7 +196,9 @@ int spg_block_sparse_attn_f16v(const int8_t *q8, const int8_t *k8, const void *v
   SPG_TRY(check_dtype(fn, out_dtype));
   SPG_NONNULL(fn, q8); SPG_NONNULL(fn, k8); SPG_NONNULL(fn, vt); SPG_NONNULL(fn, out); SPG_NONNULL(fn, lut);
   SPG_NONNULL(fn, valid_block_num); SPG_NONNULL(fn, pvthreshd); SPG_NONNULL(fn, q_scale); SPG_NONNULL(fn, k_scale);
-  return check_launch(fn, spg::launch_block_sparse_attn(q8, k8, (const uint8_t *)vt, out, out_dtype, lut, valid_block_num,
+  spg::Strides os;
+  SPG_TRY(get_strides(fn, "out_strides", out_strides, H, N, D, &os));
+  return check_launch(fn, spg::launch_block_sparse_attn(q8, k8, (const uint8_t *)vt, out, os, out_dtype, lut, valid_block_num,
                                                         pvthreshd, q_scale, k_scale, nullptr, B, H, Hkv, N, D, sm_scale,
                                                         is_causal ? 1 : 0, pv_threshold_mode, pv_count, (hipStream_t)stream));
 }

@@ -23,21 +23,21 @@ namespace spg {
 // K column mean
 // =============================================================================================
 template <int D, int DT>
-__global__ __launch_bounds__(256) void km_partial_kernel(const uint16_t *__restrict__ k, double *__restrict__ part,
-                                                         int N, int rows_per_chunk) {
+__global__ __launch_bounds__(256) void km_partial_kernel(const uint16_t *__restrict__ k, const Strides ks, int H,
+                                                         double *__restrict__ part, int N, int rows_per_chunk) {
   constexpr int TPR = D / 8;      // lanes per row (16 B each)
   constexpr int RPP = 256 / TPR;  // rows per pass of the workgroup
   const int bh = blockIdx.y, chunk = blockIdx.x, nchunk = gridDim.x;
   const int c = threadIdx.x % TPR, r = threadIdx.x / TPR;
   const int row0 = chunk * rows_per_chunk;
   const int row1 = min(N, row0 + rows_per_chunk);
-  const uint16_t *base = k + (size_t)bh * N * D + c * 8;
+  const uint16_t *base = k + (size_t)(bh / H) * ks.sb + (size_t)(bh % H) * ks.sh + c * 8;
   double acc[8];
 #pragma unroll
   for (int e = 0; e < 8; e++) acc[e] = 0.0;
 #pragma unroll 4
   for (int row = row0 + r; row < row1; row += RPP) {
-    const uint4 v = *(const uint4 *)(base + (size_t)row * D);
+    const uint4 v = *(const uint4 *)(base + (size_t)row * ks.sn);
     const uint32_t w[4] = {v.x, v.y, v.z, v.w};
 #pragma unroll
     for (int e = 0; e < 4; e++) {
@@ -112,7 +112,7 @@ __global__ __launch_bounds__(256) void div_selftest_kernel(unsigned long long *c
 }
 
 template <int BS, int D, int DT, bool HAS_MEAN, bool WITH_POOL>
-__global__ __launch_bounds__(256) void pool_sim_quant_kernel(const uint16_t *__restrict__ x,
+__global__ __launch_bounds__(256) void pool_sim_quant_kernel(const uint16_t *__restrict__ x, const Strides xs,
                                                              const uint16_t *__restrict__ km,
                                                              uint16_t *__restrict__ pool, uint8_t *__restrict__ sim,
                                                              int8_t *__restrict__ xq, float *__restrict__ scale,
@@ -124,7 +124,7 @@ __global__ __launch_bounds__(256) void pool_sim_quant_kernel(const uint16_t *__r
   const int tid = threadIdx.x, c = tid % TPR, r = tid / TPR;
   const int row_base = blk * BS;
   const int rows_valid = min(BS, N - row_base);
-  const uint16_t *xb = x + ((size_t)bh * N + row_base) * D + c * 8;
+  const uint16_t *xb = x + (size_t)(bh / H) * xs.sb + (size_t)(bh % H) * xs.sh + (size_t)row_base * xs.sn + c * 8;
 
   float kmf[8];
   if constexpr (HAS_MEAN) {
@@ -141,7 +141,7 @@ __global__ __launch_bounds__(256) void pool_sim_quant_kernel(const uint16_t *__r
   // are zeroed afterwards: no load sits behind a branch)
   uint4 raw[NP];
 #pragma unroll
-  for (int p = 0; p < NP; p++) raw[p] = *(const uint4 *)(xb + (size_t)min(r + p * RPP, rows_valid - 1) * D);
+  for (int p = 0; p < NP; p++) raw[p] = *(const uint4 *)(xb + (size_t)min(r + p * RPP, rows_valid - 1) * xs.sn);
   float xf[NP][8];
   float amax = 0.f;
 #pragma unroll
@@ -882,37 +882,37 @@ size_t km_mean_workspace_bytes(int B, int H, int N, int D) {
 }
 
 template <int D, int DT>
-static void launch_km(const void *k, void *km, void *ws, int B, int H, int N, hipStream_t st) {
+static void launch_km(const void *k, Strides ks, void *km, void *ws, int B, int H, int N, hipStream_t st) {
   const int nchunk = km_chunks(B, H, N);
   const int rpc = (N + nchunk - 1) / nchunk;
-  km_partial_kernel<D, DT><<<dim3(nchunk, B * H), 256, 0, st>>>((const uint16_t *)k, (double *)ws, N, rpc);
+  km_partial_kernel<D, DT><<<dim3(nchunk, B * H), 256, 0, st>>>((const uint16_t *)k, ks, H, (double *)ws, N, rpc);
   km_final_kernel<DT><<<B * H, D, 0, st>>>((const double *)ws, (uint16_t *)km, nchunk, D, N);
 }
 
-void launch_km_mean(const void *k, void *km, void *ws, int B, int H, int N, int D, int dtype, hipStream_t st) {
-  if (D == 64) { if (dtype == 0) launch_km<64, 0>(k, km, ws, B, H, N, st); else launch_km<64, 1>(k, km, ws, B, H, N, st); }
-  else         { if (dtype == 0) launch_km<128, 0>(k, km, ws, B, H, N, st); else launch_km<128, 1>(k, km, ws, B, H, N, st); }
+void launch_km_mean(const void *k, Strides ks, void *km, void *ws, int B, int H, int N, int D, int dtype, hipStream_t st) {
+  if (D == 64) { if (dtype == 0) launch_km<64, 0>(k, ks, km, ws, B, H, N, st); else launch_km<64, 1>(k, ks, km, ws, B, H, N, st); }
+  else         { if (dtype == 0) launch_km<128, 0>(k, ks, km, ws, B, H, N, st); else launch_km<128, 1>(k, ks, km, ws, B, H, N, st); }
 }
 
 template <int BS, int D, int DT>
-static void launch_psq3(const void *x, const void *km, void *pool, uint8_t *sim, int8_t *xq, float *scale,
+static void launch_psq3(const void *x, Strides xs, const void *km, void *pool, uint8_t *sim, int8_t *xq, float *scale,
                         const float *thr, int B, int H, int N, hipStream_t st) {
   const int nb = (N + BS - 1) / BS;
   const dim3 grid(nb, B * H);
   const uint16_t *xp = (const uint16_t *)x, *kp = (const uint16_t *)km;
   uint16_t *pp = (uint16_t *)pool;
   if (pool != nullptr) {
-    if (km) pool_sim_quant_kernel<BS, D, DT, true, true><<<grid, 256, 0, st>>>(xp, kp, pp, sim, xq, scale, thr, H, N, nb);
-    else    pool_sim_quant_kernel<BS, D, DT, false, true><<<grid, 256, 0, st>>>(xp, kp, pp, sim, xq, scale, thr, H, N, nb);
+    if (km) pool_sim_quant_kernel<BS, D, DT, true, true><<<grid, 256, 0, st>>>(xp, xs, kp, pp, sim, xq, scale, thr, H, N, nb);
+    else    pool_sim_quant_kernel<BS, D, DT, false, true><<<grid, 256, 0, st>>>(xp, xs, kp, pp, sim, xq, scale, thr, H, N, nb);
   } else {
-    if (km) pool_sim_quant_kernel<BS, D, DT, true, false><<<grid, 256, 0, st>>>(xp, kp, pp, sim, xq, scale, thr, H, N, nb);
-    else    pool_sim_quant_kernel<BS, D, DT, false, false><<<grid, 256, 0, st>>>(xp, kp, pp, sim, xq, scale, thr, H, N, nb);
+    if (km) pool_sim_quant_kernel<BS, D, DT, true, false><<<grid, 256, 0, st>>>(xp, xs, kp, pp, sim, xq, scale, thr, H, N, nb);
+    else    pool_sim_quant_kernel<BS, D, DT, false, false><<<grid, 256, 0, st>>>(xp, xs, kp, pp, sim, xq, scale, thr, H, N, nb);
   }
 }
 
-void launch_pool_sim_quant(const void *x, const void *km, void *pool, uint8_t *sim, int8_t *xq, float *scale,
+void launch_pool_sim_quant(const void *x, Strides xs, const void *km, void *pool, uint8_t *sim, int8_t *xq, float *scale,
                            const float *thr, int B, int H, int N, int D, int block, int dtype, hipStream_t st) {
-#define SPG_PSQ(BS_, D_, DT_) launch_psq3<BS_, D_, DT_>(x, km, pool, sim, xq, scale, thr, B, H, N, st)
+#define SPG_PSQ(BS_, D_, DT_) launch_psq3<BS_, D_, DT_>(x, xs, km, pool, sim, xq, scale, thr, B, H, N, st)
   if (block == 128) {
     if (D == 64) { if (dtype == 0) SPG_PSQ(128, 64, 0); else SPG_PSQ(128, 64, 1); }
     else         { if (dtype == 0) SPG_PSQ(128, 128, 0); else SPG_PSQ(128, 128, 1); }

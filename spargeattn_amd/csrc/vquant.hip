@@ -24,21 +24,21 @@ __global__ void fill_u32_kernel(uint32_t *p, uint32_t v, int n) {
 }
 
 template <int D, int DT>
-__global__ __launch_bounds__(256) void v_absmax_kernel(const uint16_t *__restrict__ v, uint32_t *__restrict__ amax_bits,
-                                                       int N, int rows_per_chunk) {
+__global__ __launch_bounds__(256) void v_absmax_kernel(const uint16_t *__restrict__ v, const Strides vs, int H,
+                                                       uint32_t *__restrict__ amax_bits, int N, int rows_per_chunk) {
   constexpr int TPR = D / 8;
   constexpr int RPP = 256 / TPR;
   const int bh = blockIdx.y, chunk = blockIdx.x;
   const int c = threadIdx.x % TPR, r = threadIdx.x / TPR;
   const int row0 = chunk * rows_per_chunk;
   const int row1 = min(N, row0 + rows_per_chunk);
-  const uint16_t *base = v + (size_t)bh * N * D + c * 8;
+  const uint16_t *base = v + (size_t)(bh / H) * vs.sb + (size_t)(bh % H) * vs.sh + c * 8;
   float m[8];
 #pragma unroll
   for (int e = 0; e < 8; e++) m[e] = 0.f;
 #pragma unroll 4
   for (int row = row0 + r; row < row1; row += RPP) {
-    const uint4 q = *(const uint4 *)(base + (size_t)row * D);
+    const uint4 q = *(const uint4 *)(base + (size_t)row * vs.sn);
     const uint32_t w[4] = {q.x, q.y, q.z, q.w};
 #pragma unroll
     for (int e = 0; e < 8; e++) {
@@ -60,8 +60,8 @@ __global__ __launch_bounds__(256) void v_absmax_kernel(const uint16_t *__restric
 
 // One workgroup per 64-key tile.  LDS holds the transposed tile [D][64] bytes.
 template <int D, int DT>
-__global__ __launch_bounds__(256) void v_quant_kernel(const uint16_t *__restrict__ v, const float *__restrict__ amax,
-                                                      uint8_t *__restrict__ v8, int N, int nk) {
+__global__ __launch_bounds__(256) void v_quant_kernel(const uint16_t *__restrict__ v, const Strides vs, int H,
+                                                      const float *__restrict__ amax, uint8_t *__restrict__ v8, int N, int nk) {
   constexpr int TPR = D / 8;
   constexpr int RPP = 256 / TPR;
   constexpr int NP = 64 / RPP;
@@ -72,11 +72,11 @@ __global__ __launch_bounds__(256) void v_quant_kernel(const uint16_t *__restrict
   float recp[8];
 #pragma unroll
   for (int e = 0; e < 8; e++) recp[e] = 2.25f / amax[(size_t)bh * D + c * 8 + e];
-  const uint16_t *base = v + ((size_t)bh * N + (size_t)blk * 64) * D + c * 8;
+  const uint16_t *base = v + (size_t)(bh / H) * vs.sb + (size_t)(bh % H) * vs.sh + (size_t)blk * 64 * vs.sn + c * 8;
   const int last_row = min(63, N - 1 - blk * 64);
   uint4 raw[NP];                     // every load is issued before the first use; rows beyond N re-read the last row
 #pragma unroll
-  for (int p = 0; p < NP; p++) raw[p] = *(const uint4 *)(base + (size_t)min(r + p * RPP, last_row) * D);
+  for (int p = 0; p < NP; p++) raw[p] = *(const uint4 *)(base + (size_t)min(r + p * RPP, last_row) * vs.sn);
 #pragma unroll
   for (int p = 0; p < NP; p++) {
     const int row = r + p * RPP;
@@ -106,8 +106,8 @@ __global__ __launch_bounds__(256) void v_quant_kernel(const uint16_t *__restrict
 // 64 keys) the eight 8-key chunks are stored at slot = chunk ^ ((d >> 1) & 7) (the LDS swizzle of the attention kernel).
 // Keys at or beyond N are zero.  One workgroup per 64-key tile.
 template <int D, int DT>
-__global__ __launch_bounds__(256) void v_tiles_f16_kernel(const uint16_t *__restrict__ v, uint16_t *__restrict__ vt,
-                                                          int N, int nk) {
+__global__ __launch_bounds__(256) void v_tiles_f16_kernel(const uint16_t *__restrict__ v, const Strides vs, int H,
+                                                          uint16_t *__restrict__ vt, int N, int nk) {
   constexpr int TPR = D / 8;
   constexpr int RPP = 256 / TPR;
   constexpr int NP = 64 / RPP;
@@ -115,11 +115,11 @@ __global__ __launch_bounds__(256) void v_tiles_f16_kernel(const uint16_t *__rest
   __shared__ __align__(16) uint16_t tile[D * LDW];
   const int blk = blockIdx.x, bh = blockIdx.y, tid = threadIdx.x;
   const int c = tid % TPR, r = tid / TPR;
-  const uint16_t *base = v + ((size_t)bh * N + (size_t)blk * 64) * D + c * 8;
+  const uint16_t *base = v + (size_t)(bh / H) * vs.sb + (size_t)(bh % H) * vs.sh + (size_t)blk * 64 * vs.sn + c * 8;
   const int last_row = min(63, N - 1 - blk * 64);
   uint4 raw[NP];
 #pragma unroll
-  for (int p = 0; p < NP; p++) raw[p] = *(const uint4 *)(base + (size_t)min(r + p * RPP, last_row) * D);
+  for (int p = 0; p < NP; p++) raw[p] = *(const uint4 *)(base + (size_t)min(r + p * RPP, last_row) * vs.sn);
 #pragma unroll
   for (int p = 0; p < NP; p++) {
     const int row = r + p * RPP;
@@ -159,30 +159,30 @@ static int v_chunks(int B, int H, int N) {
 }
 
 template <int D, int DT>
-static void launch_vq2(const void *v, uint8_t *v8, float *v_scale, int B, int H, int N, hipStream_t st) {
+static void launch_vq2(const void *v, Strides vs, uint8_t *v8, float *v_scale, int B, int H, int N, hipStream_t st) {
   const int n = B * H * D;
   const int nk = (N + 63) / 64;
   const int nchunk = v_chunks(B, H, N);
   const int rpc = (N + nchunk - 1) / nchunk;
   fill_u32_kernel<<<(n + 255) / 256, 256, 0, st>>>((uint32_t *)v_scale, 0u, n);
-  v_absmax_kernel<D, DT><<<dim3(nchunk, B * H), 256, 0, st>>>((const uint16_t *)v, (uint32_t *)v_scale, N, rpc);
-  v_quant_kernel<D, DT><<<dim3(nk, B * H), 256, 0, st>>>((const uint16_t *)v, v_scale, v8, N, nk);
+  v_absmax_kernel<D, DT><<<dim3(nchunk, B * H), 256, 0, st>>>((const uint16_t *)v, vs, H, (uint32_t *)v_scale, N, rpc);
+  v_quant_kernel<D, DT><<<dim3(nk, B * H), 256, 0, st>>>((const uint16_t *)v, vs, H, v_scale, v8, N, nk);
   v_scale_final_kernel<<<(n + 255) / 256, 256, 0, st>>>(v_scale, n);
 }
 
-void launch_v_quant_fp8(const void *v, uint8_t *v8, float *v_scale, int B, int H, int N, int D, int dtype,
+void launch_v_quant_fp8(const void *v, Strides vs, uint8_t *v8, float *v_scale, int B, int H, int N, int D, int dtype,
                         hipStream_t st) {
-  if (D == 64) { if (dtype == 0) launch_vq2<64, 0>(v, v8, v_scale, B, H, N, st); else launch_vq2<64, 1>(v, v8, v_scale, B, H, N, st); }
-  else         { if (dtype == 0) launch_vq2<128, 0>(v, v8, v_scale, B, H, N, st); else launch_vq2<128, 1>(v, v8, v_scale, B, H, N, st); }
+  if (D == 64) { if (dtype == 0) launch_vq2<64, 0>(v, vs, v8, v_scale, B, H, N, st); else launch_vq2<64, 1>(v, vs, v8, v_scale, B, H, N, st); }
+  else         { if (dtype == 0) launch_vq2<128, 0>(v, vs, v8, v_scale, B, H, N, st); else launch_vq2<128, 1>(v, vs, v8, v_scale, B, H, N, st); }
 }
 
-void launch_v_tiles_f16(const void *v, void *vt, int B, int H, int N, int D, int dtype, hipStream_t st) {
+void launch_v_tiles_f16(const void *v, Strides vs, void *vt, int B, int H, int N, int D, int dtype, hipStream_t st) {
   const int nk = (N + 63) / 64;
   const dim3 grid(nk, B * H);
   const uint16_t *vp = (const uint16_t *)v;
   uint16_t *op = (uint16_t *)vt;
-  if (D == 64) { if (dtype == 0) v_tiles_f16_kernel<64, 0><<<grid, 256, 0, st>>>(vp, op, N, nk); else v_tiles_f16_kernel<64, 1><<<grid, 256, 0, st>>>(vp, op, N, nk); }
-  else         { if (dtype == 0) v_tiles_f16_kernel<128, 0><<<grid, 256, 0, st>>>(vp, op, N, nk); else v_tiles_f16_kernel<128, 1><<<grid, 256, 0, st>>>(vp, op, N, nk); }
+  if (D == 64) { if (dtype == 0) v_tiles_f16_kernel<64, 0><<<grid, 256, 0, st>>>(vp, vs, H, op, N, nk); else v_tiles_f16_kernel<64, 1><<<grid, 256, 0, st>>>(vp, vs, H, op, N, nk); }
+  else         { if (dtype == 0) v_tiles_f16_kernel<128, 0><<<grid, 256, 0, st>>>(vp, vs, H, op, N, nk); else v_tiles_f16_kernel<128, 1><<<grid, 256, 0, st>>>(vp, vs, H, op, N, nk); }
 }
 
 }  // namespace spg

@@ -51,16 +51,24 @@ def test_argument_errors_are_reported_without_a_gpu():
     """Validation happens on the host before any launch: status code + thread-local message."""
     from spargeattn_amd import _lib
     lib = _lib.load()
-    rc = lib.spg_km_mean(None, None, None, 1, 1, 128, 96, 0, None)
+    rc = lib.spg_km_mean(None, None, None, None, 1, 1, 128, 96, 0, None)
     assert rc == _lib.SPG_ERR_UNSUPPORTED and b"head_dim" in lib.spg_last_error()
     rc = lib.spg_block_select(1, 1, 1, 1, None, None, 0, 0, 1, 1, None, 1, 1, 1, 2, 64, 0, None)
     assert rc == _lib.SPG_ERR_INVALID and b"Only one of cdfthreshd and topk" in lib.spg_last_error()
-    rc = lib.spg_pool_sim_quant(None, None, None, None, None, None, None, 1, 1, 128, 64, 128, 1, None)
+    rc = lib.spg_pool_sim_quant(None, None, None, None, None, None, None, None, 1, 1, 128, 64, 128, 1, None)
     assert rc == _lib.SPG_ERR_INVALID and b"NULL" in lib.spg_last_error()
-    rc = lib.spg_v_quant_fp8(1, 1, 1, 1, 1, 128, 64, 7, None)
+    rc = lib.spg_v_quant_fp8(1, None, 1, 1, 1, 1, 128, 64, 7, None)
     assert rc == _lib.SPG_ERR_INVALID and b"dtype" in lib.spg_last_error()
     assert lib.spg_km_mean_workspace_bytes(1, 32, 32768, 128) > 0
-    rc = lib.spg_block_sparse_attn(1, 1, 1, 1, 0, 1, 1, 1, 1, 1, 1, 1, 6, 4, 128, 64, 0.125, 0, 1, None, None)
+    rc = lib.spg_block_sparse_attn(1, 1, 1, 1, None, 0, 1, 1, 1, 1, 1, 1, 1, 6, 4, 128, 64, 0.125, 0, 1, None, None)
     assert rc == _lib.SPG_ERR_INVALID and b"must be divisible by num_kv_heads" in lib.spg_last_error()
-    rc = lib.spg_block_sparse_attn(1, 1, 1, 1, 0, 1, 1, 1, 1, 1, 1, 1, 4, 4, 128, 64, 0.125, 0, 3, None, None)
+    rc = lib.spg_block_sparse_attn(1, 1, 1, 1, None, 0, 1, 1, 1, 1, 1, 1, 1, 4, 4, 128, 64, 0.125, 0, 3, None, None)
     assert rc == _lib.SPG_ERR_INVALID and b"pv_threshold_mode" in lib.spg_last_error()
+    # strides: {batch, head, row} in elements, positive multiples of 8, row stride >= head_dim
+    import ctypes
+    bad = (ctypes.c_int64 * 3)(128 * 64, 64, 60)
+    rc = lib.spg_v_quant_fp8(1, bad, 1, 1, 1, 1, 128, 64, 0, None)
+    assert rc == _lib.SPG_ERR_INVALID and b"multiple of 8" in lib.spg_last_error()
+    bad = (ctypes.c_int64 * 3)(128 * 64, 128 * 64, 32)
+    rc = lib.spg_km_mean(1, bad, 1, 1, 1, 1, 128, 64, 0, None)
+    assert rc == _lib.SPG_ERR_INVALID and b"smaller than head_dim" in lib.spg_last_error()

@@ -133,6 +133,39 @@ def test_topk_api_end_to_end(name, shrink):
                                               vg.transpose(1, 2).contiguous(), is_causal=cfg.is_causal, topk=cfg.topk,
                                               pvthreshd=cfg.pvthreshd, tensor_layout="NHD")
     assert torch.equal(o2.transpose(1, 2), o)
+    assert o2.is_contiguous()                     # written in the caller's layout by the kernel, no copy afterwards
+
+
+def test_strided_inputs_and_output_are_read_and_written_in_place():
+    """NHD tensors, head slices of a wider tensor and a strided output buffer give the bits of the contiguous case."""
+    torch.manual_seed(3)
+    B, H, N, D = 2, 3, 448, 64
+    big = torch.randn((3, B, N, H + 2, D), device="cuda").to(torch.bfloat16)      # q, k, v interleaved with 2 spare heads
+    views = [big[i, :, :, 1:1 + H].transpose(1, 2) for i in range(3)]             # (B,H,N,D) views, row stride (H+2)*D
+    assert not any(t.is_contiguous() for t in views)
+    q, k, v = (t.contiguous() for t in views)
+    km = _lib.km_mean(k)
+    assert torch.equal(_lib.km_mean(views[1]), km)
+    thr = torch.full((H,), 0.3, device="cuda")
+    for x, xv, kmean, block in ((q, views[0], None, 128), (k, views[1], km, 64)):
+        want = _lib.pool_sim_quant(x, kmean, block, thr)
+        got = _lib.pool_sim_quant(xv, kmean, block, thr)
+        assert all(torch.equal(a, b) for a, b in zip(want, got))
+    assert all(torch.equal(a, b) for a, b in zip(_lib.v_quant_fp8(v), _lib.v_quant_fp8(views[2])))
+    assert torch.equal(_lib.v_tiles_f16_swizzled(v), _lib.v_tiles_f16_swizzled(views[2]))
+    o = sa.spas_sage2_attn_meansim_topk_cuda(q, k, v, topk=0.6)
+    o_nhd = sa.spas_sage2_attn_meansim_topk_cuda(*(big[i, :, :, 1:1 + H] for i in range(3)), topk=0.6, tensor_layout="NHD")
+    assert torch.equal(o_nhd.transpose(1, 2), o)
+    o1 = sa.spas_sage_attn_meansim_topk_cuda(q, k, v, topk=0.6, is_causal=True)
+    o1_nhd = sa.spas_sage_attn_meansim_topk_cuda(*(big[i, :, :, 1:1 + H] for i in range(3)), topk=0.6, is_causal=True,
+                                                 tensor_layout="NHD")
+    assert torch.equal(o1_nhd.transpose(1, 2), o1)
+    # rows that are not 16-byte aligned are refused by the binding and copied by the operator
+    odd = torch.randn((B, H, N, D + 4), device="cuda").to(torch.bfloat16)[..., 2:2 + D]
+    with pytest.raises(RuntimeError, match="16-byte aligned|contiguous"):
+        _lib.km_mean(odd)
+    assert torch.equal(sa.spas_sage2_attn_meansim_topk_cuda(odd, odd, odd, topk=0.6),
+                       sa.spas_sage2_attn_meansim_topk_cuda(odd.contiguous(), odd.contiguous(), odd.contiguous(), topk=0.6))
 
 
 def test_mask_api_end_to_end_cfg2_shape():
