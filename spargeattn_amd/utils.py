@@ -43,6 +43,34 @@ def get_vanilla_qk_quant(q, k, km=None, BLKQ=128, BLKK=64):
     return q_int8, q_scale, k_int8, k_scale
 
 
+def _check_block_size(block_size):
+    if block_size not in (BLKQ, BLKK):
+        raise ValueError("the gfx950 kernels pool and quantise 128-row or 64-row blocks")
+
+
+def get_quant(x, x_mean, block_size):
+    """Per-block INT8 quantisation of x, or of (x - x_mean) when the (B,H,1,D) column mean is given
+    (spas_sage_attn/utils.py:255-263): returns (x_int8, x_scale)."""
+    _check_block_size(block_size)
+    _, _, x_int8, x_scale = _lib.pool_sim_quant(x, x_mean, block_size, with_pool=False)
+    return x_int8, x_scale
+
+
+def get_pool_sim_triton_simmean_fuse_quant(x, x_mean, block_size, simthreshd1):
+    """Block means, self-similarity flags and the INT8 quantisation in one pass over x
+    (spas_sage_attn/utils.py:270-280): returns (pool, sim_blocks, x_int8, x_scale).  simthreshd1 is the (H,) float32
+    tensor hyperparameter_check returns.  The name is kept for drop-in compatibility; no Triton is involved."""
+    _check_block_size(block_size)
+    return _lib.pool_sim_quant(x, x_mean, block_size, simthreshd1)
+
+
+def get_pool_sim_triton_simmean(x, block_size, simthreshd1):
+    """Block means and self-similarity flags only (spas_sage_attn/utils.py:243-252): returns (pool, sim_blocks).
+    The fused kernel computes the quantisation as well; its int8 output is dropped."""
+    pool, sim, _, _ = get_pool_sim_triton_simmean_fuse_quant(x, None, block_size, simthreshd1)
+    return pool, sim
+
+
 def block_map_lut_triton(block_map):
     """Block map (B,H,nq,nk), non-zero = keep -> (delta LUT int32, valid_block_num int32).
 

@@ -5,7 +5,7 @@ import torch
 
 from oracle import maskpred as mp
 from oracle import vquant as vq
-from spargeattn_amd import _lib
+from spargeattn_amd import _lib, utils
 from gpu_common import tag_of, to_np, bits_equal_T, v8_natural, rand_T
 
 pytestmark = pytest.mark.gpu
@@ -168,3 +168,21 @@ def test_similarity_flag_on_degenerate_rows(dtype, thr_value):
 
 def ref_sim_128(x, thr, tag):
     return mp.pool_sim_quant(to_np(x), None, 128, thr.cpu().numpy(), tag)["sim"]
+
+
+def test_helper_wrappers_of_the_reference_utils():
+    """get_quant / get_pool_sim_triton_simmean[_fuse_quant] return what the fused stage returns (utils.py:243-280)."""
+    torch.manual_seed(11)
+    x = torch.randn((1, 2, 300, 64), device="cuda").to(torch.float16)
+    km = _lib.km_mean(x)
+    thr = utils.hyperparameter_check(0.2, 2, x.device)
+    pool, sim, xq, xs = _lib.pool_sim_quant(x, km, 64, thr)
+    got = utils.get_pool_sim_triton_simmean_fuse_quant(x, km, 64, thr)
+    assert all(torch.equal(a, b) for a, b in zip(got, (pool, sim, xq, xs)))
+    q8, qs = utils.get_quant(x, km, 64)
+    assert torch.equal(q8, xq) and torch.equal(qs, xs)
+    p2, s2 = utils.get_pool_sim_triton_simmean(x, 128, thr)
+    want = _lib.pool_sim_quant(x, None, 128, thr)
+    assert torch.equal(p2, want[0]) and torch.equal(s2, want[1])
+    with pytest.raises(ValueError):
+        utils.get_quant(x, None, 32)
