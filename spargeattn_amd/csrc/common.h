@@ -131,6 +131,16 @@ __device__ __forceinline__ double group_sum_f64(double v) {
   return v;
 }
 
+// Bitwise AND over aligned groups of G lanes (same lane permutes as group_sum_f64).
+template <int G>
+__device__ __forceinline__ uint32_t group_and_u32(uint32_t v) {
+  if constexpr (G >= 2) v &= (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0xB1, 0xf, 0xf, true);
+  if constexpr (G >= 4) v &= (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x4E, 0xf, 0xf, true);
+  if constexpr (G >= 8) v &= (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x141, 0xf, 0xf, true);
+  if constexpr (G >= 16) v &= (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x140, 0xf, 0xf, true);
+  return v;
+}
+
 __device__ __forceinline__ float wave_max_f32(float v) {
 #pragma unroll
   for (int o = 32; o >= 1; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, SPG_WAVE));

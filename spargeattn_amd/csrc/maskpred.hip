@@ -192,24 +192,43 @@ __global__ __launch_bounds__(256) void pool_sim_quant_kernel(const uint16_t *__r
     const bool sim_trivial = simthr[bh % H] < 0.f;     // workgroup-uniform
     int bad_rows = 0;
     float ssf_mine = 0.f;
+    // Column sums for the pooled mean (binary64), and - with a negative threshold - a scan of the bit patterns:
+    // only two facts about the rows are needed then, is any element non-finite and does any row have a zero norm.
+    // A row whose largest |x| is at least 2^-74 has a sum of squares of at least 2^-148, which rounds to a positive
+    // binary32 number; rows in which every element is smaller than that (all-zero rows, the padding of a partial block,
+    // bf16 values near the bottom of the range) are decided by the exact sums below.
+    uint32_t abs_max = 0, tiny_rows = 0;
 #pragma unroll
     for (int p = 0; p < NP; p++) {
-      double ss = 0.0;
+      uint32_t m = 0;
 #pragma unroll
       for (int e = 0; e < 8; e++) {
-        const double xd = (double)xf[p][e];
-        ss = __builtin_fma(xd, xd, ss);             // squares and their sum are exact in binary64
-        colsum[e] += xd;
+        colsum[e] += (double)xf[p][e];
+        m = max(m, __builtin_bit_cast(uint32_t, xf[p][e]) & 0x7fffffffu);
       }
-      ss = group_sum_f64<TPR>(ss);                 // the TPR lanes of this row
-      const float ssf = (float)ss;
-      ssf_mine = (c % NP == p) ? ssf : ssf_mine;
-      if (sim_trivial) {
-        if (!(ssf < INFINITY)) {                     // overflow of finite values is harmless (x / inf = 0); inf or NaN x is not
+      abs_max = max(abs_max, m);
+      tiny_rows |= (m < 0x1A800000u ? 1u : 0u) << p;        // 0x1A800000 = 2^-74
+    }
+    bool need_norms = true;                                  // wavefront-uniform
+    if (sim_trivial) {
+      bad_rows |= abs_max >= 0x7f800000u ? 1 : 0;           // inf or NaN anywhere (overflowing squares of finite values are harmless: x / inf = 0)
+      tiny_rows = group_and_u32<TPR>(tiny_rows);            // rows tiny in every lane of their group
+      need_norms = __any(tiny_rows != 0);                   // rare
+    }
+    if (need_norms) {
+      // sum of squares of every row (exact in binary64), rounded to binary32 like the reference's (utils.py:194)
 #pragma unroll
-          for (int e = 0; e < 8; e++) bad_rows |= __builtin_isfinite(xf[p][e]) ? 0 : 1;
+      for (int p = 0; p < NP; p++) {
+        double ss = 0.0;
+#pragma unroll
+        for (int e = 0; e < 8; e++) {
+          const double xd = (double)xf[p][e];
+          ss = __builtin_fma(xd, xd, ss);             // squares and their sum are exact in binary64
         }
-        bad_rows |= (ssf == 0.f) ? 1 : 0;
+        ss = group_sum_f64<TPR>(ss);                 // the TPR lanes of this row
+        const float ssf = (float)ss;
+        ssf_mine = (c % NP == p) ? ssf : ssf_mine;
+        if (sim_trivial) bad_rows |= (ssf == 0.f) ? 1 : 0;
       }
     }
     if (!sim_trivial) {
