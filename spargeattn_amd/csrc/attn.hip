@@ -259,10 +259,6 @@ __global__ __launch_bounds__(256, PV16 ? 2 : 3) void block_sparse_attn_kernel(co
   __syncthreads();
 #pragma unroll 1
   for (int it = 0; it < nv; it++) {
-    // scalar prefetches for later iterations (SMEM)
-    const float ksc2 = kscale[blk2];
-    const int d4 = it + 4 < nv ? lutc[it + 4] : 0;
-
     // ---- S^T = K . Q^T ---------------------------------------------------------------------------------
     SPG_LOAD_BIAS();
     {
@@ -289,6 +285,13 @@ __global__ __launch_bounds__(256, PV16 ? 2 : 3) void block_sparse_attn_kernel(co
       }
     }
 
+    // scalar prefetches for later iterations (SMEM).  Issued here, behind the last LDS wait of the products: scalar and
+    // LDS loads share one counter, so a scalar load issued at the top of the loop would be waited for together with the
+    // K operands; from here its latency runs under the MFMAs and the max reduction.
+    __builtin_amdgcn_sched_barrier(0);
+    const float ksc2 = kscale[blk2];
+    const int d4 = it + 4 < nv ? lutc[it + 4] : 0;
+    __builtin_amdgcn_sched_barrier(0);
     const float dq = qs * ksc;
     const bool tail = it >= nv - 2;   // last two blocks: masks, no PV skip (sm89.cuh:467-648)
     // S0/S1 are never rewritten (no copies at the join of the two paths): slot e < 16 is S0[e], slot e >= 16 is S1[e - 16]
