@@ -7,7 +7,8 @@
  * of thu-ml/SpargeAttn.  Every function takes raw DEVICE pointers, explicit
  * sizes, enum ints and a HIP stream (hipStream_t passed as void*); it launches
  * asynchronously on that stream, allocates nothing, synchronises nothing and
- * keeps no state.  Tensors are contiguous in the "HND" layout (B,H,N,D).
+ * keeps no state.  Tensors the library produces are contiguous (B,H,N,D) ("HND"); the caller's own q, k, v and output
+ * may be strided (see "Strides" below).
  * Return value: SPG_OK or an error code; spg_last_error() gives the message of
  * the last failure on the calling thread.
  *
@@ -63,6 +64,17 @@ size_t spg_km_mean_workspace_bytes(int B, int H, int N, int D);
 int spg_km_mean(const void *k, const int64_t *k_strides, void *km, void *workspace, int B, int H, int N, int D, int dtype,
                 void *stream);
 
+/* ---- A2 for callers that cannot allocate (no counterpart in the reference).
+ * Same result as spg_km_mean, bit for bit, without a workspace argument: the partial sums go to an 8 MiB array in
+ * device memory that the library owns (one per GPU, held until the process ends), so the call performs no allocation of
+ * any kind - it is meant for code under HIP graph capture, tight serving loops and harnesses that forbid hipMalloc.
+ * Limit: spg_km_mean_workspace_bytes(B,H,N,D) <= 8 MiB (any shape with B*H <= 8192 at D = 128 or B*H <= 16384 at D = 64);
+ * larger shapes return SPG_ERR_UNSUPPORTED.  All calls on one GPU share the array: calls that overlap in time on one
+ * GPU (two streams, two threads) race and must be ordered by the caller; calls on one stream are ordered already.
+ * The first call on a device looks the array's address up (no allocation, but make it outside a graph capture). */
+int spg_km_mean_static(const void *k, const int64_t *k_strides, void *km, int B, int H, int N, int D, int dtype,
+                       void *stream);
+
 /* ---- A3/A4: fused pool + self-similarity + per-block INT8 quantisation ------------------------
  * replaces triton_bmm_pool_sim_simmean_fuse_quant (spas_sage_attn/utils.py:161-214, wrapper 270-280).
  * x (B,H,N,D) dtype, strided; km (B,H,D) dtype or NULL (Q: NULL, K: the column mean, subtracted in dtype);
@@ -104,8 +116,10 @@ int spg_v_quant_fp8(const void *v, const int64_t *v_strides, uint8_t *v8, float 
  * (csrc/qattn/attn_cuda.h:61-76, csrc/qattn/qk_int_sv_f8_cuda_sm89.cu:197-390) with
  * tensor_layout = HND, qk_quant_gran = per-block; pv_threshold_mode = SPG_PV_PER_BLOCK is what that entry point
  * compiles in (sm89.cu:365), the other two modes are the kernel template's (sm89.cuh:283-391).
- * q8 int8 (B,H,N,D); k8 int8 (B,Hkv,N,D); v8 as produced by spg_v_quant_fp8 for Hkv heads; out (B,H,N,D) out_dtype, strided;
- * lut/valid_block_num as above; pvthreshd (H,) float32; q_scale (B,H,nq), k_scale (B,Hkv,nk),
+ * q8 int8 (B,H,N,D); k8 int8 (B,Hkv,N_kv,D); v8 as produced by spg_v_quant_fp8 for Hkv heads of N_kv rows; out (B,H,N,D)
+ * out_dtype, strided.  N (qo_len) and N_kv (kv_len) are independent as in the reference (sm89.cu:256-300):
+ * nq = ceil(N/128), nk = ceil(N_kv/64); keys >= N_kv of the last block are masked.
+ * lut (B,H,nq,nk) / valid_block_num as above; pvthreshd (H,) float32; q_scale (B,H,nq), k_scale (B,Hkv,nk),
  * v_scale (B,Hkv,D) float32; Hkv divides H: query head h reads K/V head h / (H / Hkv) (grouped-query attention,
  * sm89.cu:310-314, sm89.cuh:118); Hkv = H is plain multi-head attention; pv_count (B,H,nq*4) int32 or NULL: number of K blocks
  * whose PV was computed, one entry per 32 query rows as in the reference (sm89.cu:331-334); entries of Q blocks with
@@ -114,8 +128,8 @@ int spg_v_quant_fp8(const void *v, const int64_t *v_strides, uint8_t *v8, float 
 int spg_block_sparse_attn(const int8_t *q8, const int8_t *k8, const uint8_t *v8, void *out, const int64_t *out_strides,
                           int out_dtype, const int32_t *lut, const int32_t *valid_block_num, const float *pvthreshd,
                           const float *q_scale, const float *k_scale, const float *v_scale,
-                          int B, int H, int Hkv, int N, int D, float sm_scale, int is_causal, int pv_threshold_mode,
-                          int32_t *pv_count, void *stream);
+                          int B, int H, int Hkv, int N, int N_kv, int D, float sm_scale, int is_causal,
+                          int pv_threshold_mode, int32_t *pv_count, void *stream);
 
 /* ---- SageAttention1-style variant: INT8 QK^T, FP16 PV.
  * Replaces qk_int8_sv_f16_accum_f16_block_sparse_attn_inst_buf_with_pv_threshold (csrc/qattn/attn_cuda.h:32-45,
@@ -130,8 +144,8 @@ int spg_v_tiles_f16(const void *v, const int64_t *v_strides, void *vt, int B, in
 int spg_block_sparse_attn_f16v(const int8_t *q8, const int8_t *k8, const void *vt, void *out, const int64_t *out_strides,
                                int out_dtype, const int32_t *lut, const int32_t *valid_block_num, const float *pvthreshd,
                                const float *q_scale, const float *k_scale,
-                               int B, int H, int Hkv, int N, int D, float sm_scale, int is_causal, int pv_threshold_mode,
-                               int32_t *pv_count, void *stream);
+                               int B, int H, int Hkv, int N, int N_kv, int D, float sm_scale, int is_causal,
+                               int pv_threshold_mode, int32_t *pv_count, void *stream);
 
 /* ---- measurement comparator: dense FP16 flash attention on MFMA (no counterpart in the reference;
  * the "dense FP16 attention kernel built in the same run" the speed-up is quoted against).
@@ -144,6 +158,12 @@ int spg_dense_attn_f16(const void *q, const void *k, const void *vt, void *out, 
  * hardware's correctly rounded one for every finite fp16 and bf16 numerator against n_divisors pseudo-random
  * divisors.  counts (device, 2 x uint64, zeroed by the caller): [0] += comparisons, [1] += mismatches. */
 int spg_selftest_division(unsigned long long *counts, int n_divisors, unsigned int seed, void *stream);
+
+/* ---- self test (no counterpart in the reference): the fp32 -> e4m3 pack of the probabilities.
+ * x (n,) float32 device, n a multiple of 4 -> codes (n,) uint8.  saturate != 0: exactly what spg_block_sparse_attn does
+ * (round to nearest even, |x| > 448 clamps to +-448 like cvt.rn.satfinite.e4m3x2.f32, csrc/numeric_conversion.cuh:48-63);
+ * saturate == 0: the bare v_cvt_pk_fp8_f32 instruction, for documentation of what the hardware does without the clamp. */
+int spg_selftest_fp8_pack(const float *x, uint8_t *codes, int n, int saturate, void *stream);
 
 #ifdef __cplusplus
 }

@@ -25,15 +25,17 @@ SIGNATURES = {
     "spg_last_error": (_c.c_char_p, []),
     "spg_km_mean_workspace_bytes": (_sz, [_i, _i, _i, _i]),
     "spg_km_mean": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp]),
+    "spg_km_mean_static": (_i, [_vp, _vp, _vp, _i, _i, _i, _i, _i, _vp]),
     "spg_pool_sim_quant": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp]),
     "spg_block_select": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp]),
     "spg_map_to_lut": (_i, [_vp, _i, _vp, _vp, _i, _i, _i, _i, _vp]),
     "spg_v_quant_fp8": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp]),
-    "spg_block_sparse_attn": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _f, _i, _i, _vp, _vp]),
+    "spg_block_sparse_attn": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _f, _i, _i, _vp, _vp]),
     "spg_v_tiles_f16": (_i, [_vp, _vp, _vp, _i, _i, _i, _i, _i, _vp]),
-    "spg_block_sparse_attn_f16v": (_i, [_vp] * 5 + [_i] + [_vp] * 5 + [_i] * 5 + [_f, _i, _i, _vp, _vp]),
+    "spg_block_sparse_attn_f16v": (_i, [_vp] * 5 + [_i] + [_vp] * 5 + [_i] * 6 + [_f, _i, _i, _vp, _vp]),
     "spg_dense_attn_f16": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _f, _i, _vp]),
     "spg_selftest_division": (_i, [_vp, _i, ctypes.c_uint, _vp]),
+    "spg_selftest_fp8_pack": (_i, [_vp, _vp, _i, _i, _vp]),
 }
 
 _lib = None
@@ -214,14 +216,38 @@ def v8_natural_to_tiles(v8_nat):
 PV_NONE, PV_PER_BLOCK, PV_PER_WARP = 0, 1, 2
 
 
+def _check_attn_shapes(q8, k8, vt, lut, valid, q_scale, k_scale, v_scale=None):
+    """Shapes the attention kernels index with: raises before a launch could read past a buffer.
+    The query length N and the key/value length N_kv are independent (qo_len / kv_len of
+    csrc/qattn/qk_int_sv_f8_cuda_sm89.cu:256-300)."""
+    B, H, N, D = q8.shape
+    Hkv, Nk = k8.shape[1], k8.shape[2]
+    nq, nk = (N + 127) // 128, (Nk + 63) // 64
+    if k8.shape[0] != B or k8.shape[3] != D:
+        raise RuntimeError(f"k shape {tuple(k8.shape)} does not match q shape {tuple(q8.shape)}")
+    if tuple(vt.shape) != (B, Hkv, nk, D, 64):
+        raise RuntimeError(f"V tiles have shape {tuple(vt.shape)}, expected {(B, Hkv, nk, D, 64)} for kv_len {Nk}")
+    if tuple(lut.shape) != (B, H, nq, nk) or tuple(valid.shape) != (B, H, nq):
+        raise RuntimeError(f"lut / valid_block_num have shapes {tuple(lut.shape)} / {tuple(valid.shape)}, "
+                           f"expected {(B, H, nq, nk)} / {(B, H, nq)}")
+    if tuple(q_scale.shape) != (B, H, nq) or tuple(k_scale.shape) != (B, Hkv, nk):
+        raise RuntimeError(f"q_scale / k_scale have shapes {tuple(q_scale.shape)} / {tuple(k_scale.shape)}, "
+                           f"expected {(B, H, nq)} / {(B, Hkv, nk)}")
+    if v_scale is not None and tuple(v_scale.shape) != (B, Hkv, D):
+        raise RuntimeError(f"v_scale has shape {tuple(v_scale.shape)}, expected {(B, Hkv, D)}")
+    return B, H, Hkv, N, Nk, D
+
+
 def block_sparse_attn(q8, k8, v8, out, lut, valid, pvthreshd, q_scale, k_scale, v_scale, sm_scale,
                       is_causal=False, return_pv_count=False, pv_mode=PV_PER_BLOCK):
     _dev(q8, k8, v8, lut, valid, pvthreshd, q_scale, k_scale, v_scale)
     _dev_strided(out)
-    B, H, N, D = q8.shape
+    B, H, Hkv, N, Nk, D = _check_attn_shapes(q8, k8, v8, lut, valid, q_scale, k_scale, v_scale)
+    if tuple(out.shape) != (B, H, N, D) or pvthreshd.numel() != H:
+        raise RuntimeError("out must have q's shape and pvthreshd one entry per query head")
     pvc = torch.zeros((B, H, 4 * ((N + 127) // 128)), dtype=torch.int32, device=q8.device) if return_pv_count else None
     _check(load().spg_block_sparse_attn(_p(q8), _p(k8), _p(v8), _p(out), _st(out), _dt(out), _p(lut), _p(valid), _p(pvthreshd),
-                                        _p(q_scale), _p(k_scale), _p(v_scale), B, H, k8.shape[1], N, D, float(sm_scale),
+                                        _p(q_scale), _p(k_scale), _p(v_scale), B, H, Hkv, N, Nk, D, float(sm_scale),
                                         int(bool(is_causal)), int(pv_mode), _p(pvc), _stream()))
     return pvc
 
@@ -250,10 +276,12 @@ def block_sparse_attn_f16v(q8, k8, vt, out, lut, valid, pvthreshd, q_scale, k_sc
                            return_pv_count=False, pv_mode=PV_PER_BLOCK):
     _dev(q8, k8, vt, lut, valid, pvthreshd, q_scale, k_scale)
     _dev_strided(out)
-    B, H, N, D = q8.shape
+    B, H, Hkv, N, Nk, D = _check_attn_shapes(q8, k8, vt, lut, valid, q_scale, k_scale)
+    if tuple(out.shape) != (B, H, N, D) or pvthreshd.numel() != H:
+        raise RuntimeError("out must have q's shape and pvthreshd one entry per query head")
     pvc = torch.zeros((B, H, 4 * ((N + 127) // 128)), dtype=torch.int32, device=q8.device) if return_pv_count else None
     _check(load().spg_block_sparse_attn_f16v(_p(q8), _p(k8), _p(vt), _p(out), _st(out), _dt(out), _p(lut), _p(valid),
-                                             _p(pvthreshd), _p(q_scale), _p(k_scale), B, H, k8.shape[1], N, D, float(sm_scale),
+                                             _p(pvthreshd), _p(q_scale), _p(k_scale), B, H, Hkv, N, Nk, D, float(sm_scale),
                                              int(bool(is_causal)), int(pv_mode), _p(pvc), _stream()))
     return pvc
 
@@ -277,6 +305,15 @@ def dense_attn_f16(q, k, vt, sm_scale, is_causal=False, out=None):
     _check(load().spg_dense_attn_f16(_p(q), _p(k), _p(vt), _p(out), B, H, N, D, float(sm_scale),
                                      int(bool(is_causal)), _stream()))
     return out
+
+
+def selftest_fp8_pack(x, saturate=True):
+    """float32 GPU tensor (size a multiple of 4) -> uint8 e4m3 codes from the attention kernel's pack."""
+    _dev(x)
+    assert x.dtype == torch.float32 and x.numel() % 4 == 0
+    codes = torch.empty(x.numel(), dtype=torch.uint8, device=x.device)
+    _check(load().spg_selftest_fp8_pack(_p(x), _p(codes), x.numel(), int(bool(saturate)), _stream()))
+    return codes.view(x.shape)
 
 
 def selftest_division(n_divisors, seed=1):

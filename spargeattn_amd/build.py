@@ -27,17 +27,41 @@ SOURCES = {
     "dense.hip": [],
     "capi.hip": ["-fvisibility=default"],
 }
+# Translation units whose kernels read LDS through inline asm into registers the compiler believes are already
+# written: a spill or a scratch copy between such a read and its wait would store stale data, so the build fails
+# when any kernel of these files uses scratch memory or spills a register.
+NO_SPILL = {"attn.hip", "dense.hip"}
+RESOURCE_REMARKS = "-Rpass-analysis=kernel-resource-usage"
+
+
+def _spill_report(stderr):
+    """Kernel names of a -Rpass-analysis=kernel-resource-usage log that use scratch or spill registers."""
+    bad, name = [], None
+    for line in stderr.splitlines():
+        if "Function Name:" in line:
+            name = line.split("Function Name:")[1].split("[")[0].strip()
+        for key in ("ScratchSize [bytes/lane]:", "SGPRs Spill:", "VGPRs Spill:"):
+            if key in line:
+                value = line.split(key)[1].split("[")[0].strip()
+                if value != "0":
+                    bad.append(f"{name}: {key} {value}")
+    return bad
 
 
 def _compile(item):
     src, extra = item
     obj = os.path.join(CSRC, src.replace(".hip", ".o"))
-    cmd = [HIPCC, *COMMON, *extra, "-c", os.path.join(CSRC, src), "-o", obj]
+    guard = [RESOURCE_REMARKS, "-fno-caret-diagnostics"] if src in NO_SPILL else []
+    cmd = [HIPCC, *COMMON, *extra, *guard, "-c", os.path.join(CSRC, src), "-o", obj]
     r = subprocess.run(cmd, capture_output=True, text=True)
-    noise = "is not a recognized feature for this target"
-    err = "\n".join(l for l in r.stderr.splitlines() if noise not in l)
+    noise = ("is not a recognized feature for this target", RESOURCE_REMARKS)
+    err = "\n".join(l for l in r.stderr.splitlines() if not any(n in l for n in noise))
     if r.returncode != 0:
         raise RuntimeError(f"hipcc failed for {src}:\n{' '.join(cmd)}\n{err}")
+    if guard:
+        bad = _spill_report(r.stderr)
+        if bad:
+            raise RuntimeError(f"{src}: kernels must not spill or use scratch memory:\n  " + "\n  ".join(bad))
     return obj, err
 
 

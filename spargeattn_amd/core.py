@@ -36,6 +36,13 @@ def _prologue(q, k, v, tensor_layout):
         q, k, v = (t.transpose(-2, -3) for t in (q, k, v))
     assert q.size(-2) >= 128, "seq_len should be not less than 128."
     assert q.size(-1) in [64, 128], "headdim should be in [64, 128]. For other headdim, you can use padding and specify the softmax scale."
+    # q may be shorter or longer than k/v (qo_len / kv_len of csrc/qattn/qk_int_sv_f8_cuda_sm89.cu:256-300); k and v
+    # must agree with each other and with q in batch and head_dim, which the reference's kernel entry checks
+    # (CHECK_SHAPE, sm89.cu:339-363 -> RuntimeError)
+    if (q.dim() != 4 or k.dim() != 4 or v.dim() != 4 or k.shape[:3] != v.shape[:3] or k.size(0) != q.size(0)
+            or k.size(-1) != q.size(-1) or v.size(-1) != q.size(-1)):
+        raise RuntimeError(f"inconsistent shapes: q {tuple(q.shape)}, k {tuple(k.shape)}, v {tuple(v.shape)} "
+                           "(as (B,H,N,D): k and v must have the same batch, heads and length, and q's batch and head_dim)")
     if not v.is_cuda:
         raise RuntimeError("spargeattn_amd needs GPU tensors (there is no CPU path)")
     torch.cuda.set_device(v.device)
@@ -56,8 +63,10 @@ def _prologue(q, k, v, tensor_layout):
 def _rows_ok(t):
     """t itself if the strided kernels can read it (last dimension contiguous, 16-byte aligned rows), else a copy."""
     esz = t.element_size()
+    # a stride of 0 (an expanded / broadcast view) or a negative one is not something the kernels take: copy, as the
+    # reference does for every input (core.py:113-117)
     ok = (t.stride(-1) == 1 and t.data_ptr() % 16 == 0 and t.dtype in (torch.float16, torch.bfloat16)
-          and all((st * esz) % 16 == 0 for st in t.stride()[:-1]))
+          and all(st > 0 and (st * esz) % 16 == 0 for st in t.stride()[:-1]))
     return t if ok else t.contiguous()
 
 

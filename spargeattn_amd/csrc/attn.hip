@@ -50,7 +50,7 @@ struct AttnParams {
   const int32_t *lut, *valid;
   const float *pvthr, *q_scale, *k_scale, *v_scale;
   int32_t *pv_count;
-  int B, H, Hkv, N, nq, nk;
+  int B, H, Hkv, N, Nk, nq, nk;   // N query rows, Nk key/value rows per head (qo_len / kv_len of sm89.cu:256-300)
   float sm_scale_log2;
   int is_causal;
   int pv_mode;     // PVThresholdMode of the reference (attn_utils.cuh:58-62): 0 none, 1 per block, 2 per wavefront of 32 rows
@@ -74,6 +74,38 @@ __device__ __forceinline__ void lds_wait4(v4i &a, v4i &b, v4i &c, v4i &d) {
 }
 __device__ __forceinline__ void lds_wait2(v4i &a, v4i &b) { asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(a), "+v"(b)); }
 __device__ __forceinline__ void lds_wait_acc(v16i &a, v16i &b) { asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(a), "+v"(b)); }
+
+// e4m3 pack of the probabilities.  v_cvt_pk_fp8_f32 returns NaN (0x7f) for |x| > 464 unless MODE.FP16_OVFL is set, in
+// which case it clamps to +-448 like the reference's cvt.rn.satfinite.e4m3x2.f32 (csrc/numeric_conversion.cuh:48-63);
+// the bit is set once per wavefront, costs nothing per element and affects no other instruction this kernel depends on
+// (the fp16 epilogue conversion cannot overflow: |O / d| <= max |V|).
+__device__ __forceinline__ void fp8_saturation_on() {
+  __builtin_amdgcn_s_setreg(1 | (23 << 6) | (0 << 11), 1);   // hwreg(HW_REG_MODE, offset 23, size 1) = FP16_OVFL
+}
+__device__ __forceinline__ int pack4_e4m3(float x0, float x1, float x2, float x3) {
+  // both halves of the destination are written, so its initial content is irrelevant: start from a register that is
+  // "defined" by an empty asm instead of a zeroed one
+  int wv;
+  asm volatile("" : "=v"(wv));
+  wv = __builtin_amdgcn_cvt_pk_fp8_f32(x0, x1, wv, false);
+  wv = __builtin_amdgcn_cvt_pk_fp8_f32(x2, x3, wv, true);
+  return wv;
+}
+
+// Self test of the pack: codes[i] = e4m3(x[i]) exactly as the attention kernel produces it (saturate != 0) or as the bare
+// instruction does (saturate == 0).  n is a multiple of 4.
+__global__ __launch_bounds__(256) void fp8_pack_selftest_kernel(const float *__restrict__ x, uint32_t *__restrict__ codes,
+                                                                int n4, int saturate) {
+  if (saturate) fp8_saturation_on();
+  const int i = blockIdx.x * 256 + threadIdx.x;
+  if (i >= n4) return;
+  const float4 v = ((const float4 *)x)[i];
+  codes[i] = (uint32_t)pack4_e4m3(v.x, v.y, v.z, v.w);
+}
+void launch_fp8_pack_selftest(const float *x, uint8_t *codes, int n, int saturate, hipStream_t st) {
+  const int n4 = n / 4;
+  fp8_pack_selftest_kernel<<<(n4 + 255) / 256, 256, 0, st>>>(x, (uint32_t *)codes, n4, saturate);
+}
 
 // 16-byte-chunk swizzles.  K tile row = key (D bytes, D/16 chunks); V^T tile row = channel (64 bytes, 4 chunks).
 // The LDS serves a ds_read_b128 one half-wavefront (32 lanes) at a time and needs two clocks for it when the 32
@@ -131,9 +163,10 @@ __global__ __launch_bounds__(256, PV16 ? 2 : 3) void block_sparse_attn_kernel(co
 
   const int tid = threadIdx.x, lane = tid & 63, r = lane & 31, hh = lane >> 5;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);   // uniform: everything derived from it stays scalar
-  const int N = p.N;
+  const int N = p.N, Nk = p.Nk;
   const int q_row = qb * 128 + wave * 32 + r;
   if (tid < 4) sBias[tid] = SPG_ACC_BIAS_BITS;   // visible after the barrier that precedes the loop
+  if constexpr (!PV16) fp8_saturation_on();
 
   // ---- Q fragment: B operand of S^T = K.Q^T, resident for the whole loop -------------------------------
   v4i qreg[KS];
@@ -143,7 +176,7 @@ __global__ __launch_bounds__(256, PV16 ? 2 : 3) void block_sparse_attn_kernel(co
     if (q_row < N) qreg[ks] = *(const v4i *)(p.q8 + ((size_t)bh * N + q_row) * D + 32 * ks + 16 * hh);
   }
 
-  const int8_t *kbase = p.k8 + (size_t)bhk * N * D;
+  const int8_t *kbase = p.k8 + (size_t)bhk * Nk * D;
   const uint8_t *vbase = p.v8 + (size_t)bhk * p.nk * (size_t)VTILE;
   // LUT and K scales are read through the constant address space: uniform addresses become scalar loads (SMEM),
   // which never touch the vector-memory counter the tile ring is synchronised with.
@@ -167,7 +200,7 @@ __global__ __launch_bounds__(256, PV16 ? 2 : 3) void block_sparse_attn_kernel(co
   const uint32_t pos0 = (uint32_t)(WL * 64 * wave) + lane_;                                                   \
   const uint32_t v_lane = ((uint32_t)(WLV * 64 * wave) + lane_) * 16u;                                        \
   const uint32_t k_lane = (pos0 * 16u) ^ (k_swz<D>(pos0 / CPR) * 16u);   /* row * D + (slot ^ swz) * 16 */
-  const int last_partial_blk = (N % 64) ? p.nk - 1 : -1;   // the only block with rows beyond N
+  const int last_partial_blk = (Nk % 64) ? p.nk - 1 : -1;   // the only block with rows beyond Nk
   typedef __attribute__((address_space(3))) void *lds_ptr_t;
   typedef const __attribute__((address_space(1))) void *glb_ptr_t;
 #define SPG_LOAD_TILES(BLK, BUFOFF)                                                                           \
@@ -189,8 +222,8 @@ __global__ __launch_bounds__(256, PV16 ? 2 : 3) void block_sparse_attn_kernel(co
         __builtin_amdgcn_global_load_lds((glb_ptr_t)(vb_ + v_lane), (lds_ptr_t)lv_, 16, 3072, 0);             \
       }                                                                                                       \
     } else {                                                                                                  \
-      /* rows beyond N are clamped to row N-1: their scores are masked, their V rows are zero */              \
-      const int rows_ok_ = N - (BLK) * 64;                                                                    \
+      /* rows beyond Nk are clamped to row Nk-1: their scores are masked, their V rows are zero */              \
+      const int rows_ok_ = Nk - (BLK) * 64;                                                                    \
       _Pragma("unroll") for (int u = 0; u < WL; u++) {                                                        \
         const uint32_t pos = pos0 + u * 64;                                                                   \
         const uint32_t row_ = min(pos / CPR, (uint32_t)(rows_ok_ - 1));                                       \
@@ -296,12 +329,18 @@ __global__ __launch_bounds__(256, PV16 ? 2 : 3) void block_sparse_attn_kernel(co
     const bool tail = it >= nv - 2;   // last two blocks: masks, no PV skip (sm89.cuh:467-648)
     // S0/S1 are never rewritten (no copies at the join of the two paths): slot e < 16 is S0[e], slot e >= 16 is S1[e - 16]
     const float a = c * dq;
-    float fm;
+    // The accumulator bias leaves the exponent through ONE additive constant, -(12582912 a + m) (+ 8.807), whose rounding
+    // error is half an ulp of 12582912 a.  Below 2^14 that is at most 2^-11 in the exponent (3e-4 relative in P, and the
+    // row maximum's P stays below 448.2).  At or above it (large |q| |k| or a large softmax scale; uniform for the
+    // workgroup) the scores are first taken relative to the lane's own maximum - an exact subtraction inside one binade -
+    // so that no large constant is left to round: one more instruction per score, on such blocks only.
+    const bool precise = a * SPG_ACC_BIAS >= 16384.0f;
+    float fm, mloc = SPG_ACC_BIAS;
     auto tail_limit = [&]() {
       const int key0 = blk * 64 + 32 * hh;
       int lim = 0x7fffffff;
       if (p.is_causal) lim = q_row - key0;                       // key > query (attn_utils.cuh:334-361)
-      if (it == nv - 1) lim = min(lim, N - 1 - key0);            // key >= kv_len (attn_utils.cuh:363-389)
+      if (it == nv - 1) lim = min(lim, Nk - 1 - key0);            // key >= kv_len (attn_utils.cuh:363-389)
       return lim;
     };
     if (!tail) {
@@ -311,6 +350,7 @@ __global__ __launch_bounds__(256, PV16 ? 2 : 3) void block_sparse_attn_kernel(co
 #pragma unroll
       for (int e = 0; e < 16; e++) imax = max(imax, S1[e]);
       fm = (float)(imax - SPG_ACC_BIAS_BITS) * a;
+      mloc = __builtin_bit_cast(float, imax);   // 12582912 + the largest of this lane's 32 dot products
     } else {
       // slot e of this lane is key 64*blk + 32*hh + e; keys beyond `lim` are masked
       const int lim = tail_limit();
@@ -358,14 +398,23 @@ __global__ __launch_bounds__(256, PV16 ? 2 : 3) void block_sparse_attn_kernel(co
     if (compute) {
       cnt++;
       const float neg0 = PV16 ? -m : -m + SPG_FP8_OFFSET;
-      const float neg = __builtin_fmaf(-SPG_ACC_BIAS, a, neg0);   // takes the accumulator bias out: one rounding per row
       float ps = 0.f;
       float x[32];
       if (!tail) {
         // three passes kept apart for the scheduler: a multiply-add feeding the exponential of the same element directly,
         // and the exponential feeding the running sum, would issue as one long chain of dependent instructions
+        if (!precise) {
+          const float neg = __builtin_fmaf(-SPG_ACC_BIAS, a, neg0);   // takes the accumulator bias out: one rounding per row
 #pragma unroll
-        for (int e = 0; e < 32; e++) x[e] = __builtin_fmaf(__builtin_bit_cast(float, e < 16 ? S0[e] : S1[e - 16]), a, neg);
+          for (int e = 0; e < 32; e++) x[e] = __builtin_fmaf(__builtin_bit_cast(float, e < 16 ? S0[e] : S1[e - 16]), a, neg);
+        } else {
+          // (S - S_max,lane) a + (S_max,lane a - m + offset): what the reference's fma(S, a, -m + offset) computes
+          // (attn_utils.cuh:391-415), with the rounding of m as the only error
+          const float c0 = __builtin_fmaf(mloc - SPG_ACC_BIAS, a, neg0);
+#pragma unroll
+          for (int e = 0; e < 32; e++)
+            x[e] = __builtin_fmaf(__builtin_bit_cast(float, e < 16 ? S0[e] : S1[e - 16]) - mloc, a, c0);
+        }
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int e = 0; e < 32; e++) x[e] = __builtin_amdgcn_exp2f(x[e]);
@@ -379,7 +428,9 @@ __global__ __launch_bounds__(256, PV16 ? 2 : 3) void block_sparse_attn_kernel(co
         const float masked = __builtin_fmaf(SPG_NEG_BIG, c, neg0);   // what the sentinel score turns into
 #pragma unroll
         for (int e = 0; e < 32; e++) {
-          const float t = __builtin_fmaf(__builtin_bit_cast(float, e < 16 ? S0[e] : S1[e - 16]), a, neg);
+          // de-quantised score first, then the softmax scale, as the reference's masked branch does (sm89.cuh:467-648)
+          const float sv = (__builtin_bit_cast(float, e < 16 ? S0[e] : S1[e - 16]) - SPG_ACC_BIAS) * dq;
+          const float t = __builtin_fmaf(sv, c, neg0);
           x[e] = __builtin_amdgcn_exp2f(e > lim ? masked : t);
           if constexpr (!PV16) ps += x[e];
         }
@@ -440,15 +491,7 @@ __global__ __launch_bounds__(256, PV16 ? 2 : 3) void block_sparse_attn_kernel(co
       dsum += ps;
       v8i pb;
 #pragma unroll
-      for (int u = 0; u < 8; u++) {
-        // both halves of the destination are written, so its initial content is irrelevant: start from a register
-        // that is "defined" by an empty asm instead of a zeroed one
-        int wv;
-        asm volatile("" : "=v"(wv));
-        wv = __builtin_amdgcn_cvt_pk_fp8_f32(x[4 * u], x[4 * u + 1], wv, false);
-        wv = __builtin_amdgcn_cvt_pk_fp8_f32(x[4 * u + 2], x[4 * u + 3], wv, true);
-        pb[u] = wv;
-      }
+      for (int u = 0; u < 8; u++) pb[u] = pack4_e4m3(x[4 * u], x[4 * u + 1], x[4 * u + 2], x[4 * u + 3]);
       {
         constexpr int HD = NDT / 2;
         const uint32_t va_lo = lds_v0 + bufoff + v_rd_lo, va_hi = lds_v0 + bufoff + (v_rd_lo ^ 16u);
@@ -518,12 +561,12 @@ __global__ __launch_bounds__(256, PV16 ? 2 : 3) void block_sparse_attn_kernel(co
 hipError_t launch_block_sparse_attn(const int8_t *q8, const int8_t *k8, const uint8_t *v8, void *out, Strides os,
                                     int out_dtype, const int32_t *lut, const int32_t *valid, const float *pvthreshd,
                                     const float *q_scale, const float *k_scale, const float *v_scale, int B, int H,
-                                    int Hkv, int N, int D, float sm_scale, int is_causal, int pv_mode,
+                                    int Hkv, int N, int Nk, int D, float sm_scale, int is_causal, int pv_mode,
                                     int32_t *pv_count, hipStream_t st) {
   AttnParams p;
   p.q8 = q8; p.k8 = k8; p.v8 = v8; p.out = out; p.os = os; p.lut = lut; p.valid = valid; p.pvthr = pvthreshd;
   p.q_scale = q_scale; p.k_scale = k_scale; p.v_scale = v_scale; p.pv_count = pv_count;
-  p.B = B; p.H = H; p.Hkv = Hkv; p.N = N; p.nq = (N + 127) / 128; p.nk = (N + 63) / 64;
+  p.B = B; p.H = H; p.Hkv = Hkv; p.N = N; p.Nk = Nk; p.nq = (N + 127) / 128; p.nk = (Nk + 63) / 64;
   p.sm_scale_log2 = sm_scale * SPG_LOG2E;
   p.is_causal = is_causal;
   p.pv_mode = pv_mode;

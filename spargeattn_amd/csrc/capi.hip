@@ -90,6 +90,20 @@ int spg_km_mean(const void *k, const int64_t *k_strides, void *km, void *workspa
   return check_launch(fn, hipSuccess);
 }
 
+int spg_km_mean_static(const void *k, const int64_t *k_strides, void *km, int B, int H, int N, int D, int dtype, void *stream) {
+  const char *fn = "spg_km_mean_static";
+  SPG_TRY(check_shape(fn, B, H, N, D));
+  SPG_TRY(check_dtype(fn, dtype));
+  SPG_NONNULL(fn, k); SPG_NONNULL(fn, km);
+  const size_t need = spg::km_mean_workspace_bytes(B, H, N, D);
+  if (need > spg::km_mean_static_capacity())
+    return fail(SPG_ERR_UNSUPPORTED, "%s: B=%d H=%d N=%d D=%d needs %zu bytes of scratch, the built-in array holds %zu "
+                "(use spg_km_mean with a workspace of your own)", fn, B, H, N, D, need, spg::km_mean_static_capacity());
+  spg::Strides ks;
+  SPG_TRY(get_strides(fn, "k_strides", k_strides, H, N, D, &ks));
+  return check_launch(fn, spg::launch_km_mean_static(k, ks, km, B, H, N, D, dtype, (hipStream_t)stream));
+}
+
 int spg_pool_sim_quant(const void *x, const int64_t *x_strides, const void *km, void *pool, uint8_t *sim, int8_t *xq, float *scale,
                        const float *simthreshd1, int B, int H, int N, int D, int block, int dtype, void *stream) {
   const char *fn = "spg_pool_sim_quant";
@@ -142,6 +156,14 @@ int spg_selftest_division(unsigned long long *counts, int n_divisors, unsigned i
   return check_launch(fn, hipSuccess);
 }
 
+int spg_selftest_fp8_pack(const float *x, uint8_t *codes, int n, int saturate, void *stream) {
+  const char *fn = "spg_selftest_fp8_pack";
+  if (n <= 0 || n % 4 != 0) return fail(SPG_ERR_INVALID, "%s: n must be a positive multiple of 4 (got %d)", fn, n);
+  SPG_NONNULL(fn, x); SPG_NONNULL(fn, codes);
+  spg::launch_fp8_pack_selftest(x, codes, n, saturate ? 1 : 0, (hipStream_t)stream);
+  return check_launch(fn, hipSuccess);
+}
+
 int spg_v_quant_fp8(const void *v, const int64_t *v_strides, uint8_t *v8, float *v_scale, int B, int H, int N, int D, int dtype, void *stream) {
   const char *fn = "spg_v_quant_fp8";
   SPG_TRY(check_shape(fn, B, H, N, D));
@@ -157,9 +179,10 @@ int spg_block_sparse_attn(const int8_t *q8, const int8_t *k8, const uint8_t *v8,
                           int out_dtype,
                           const int32_t *lut, const int32_t *valid_block_num, const float *pvthreshd,
                           const float *q_scale, const float *k_scale, const float *v_scale, int B, int H, int Hkv, int N,
-                          int D, float sm_scale, int is_causal, int pv_threshold_mode, int32_t *pv_count, void *stream) {
+                          int N_kv, int D, float sm_scale, int is_causal, int pv_threshold_mode, int32_t *pv_count, void *stream) {
   const char *fn = "spg_block_sparse_attn";
   SPG_TRY(check_shape(fn, B, H, N, D));
+  SPG_TRY(check_shape(fn, B, Hkv > 0 ? Hkv : 1, N_kv, D));
   SPG_TRY(check_kv_heads(fn, H, Hkv));
   SPG_TRY(check_pv_mode(fn, pv_threshold_mode));
   SPG_TRY(check_dtype(fn, out_dtype));
@@ -169,7 +192,7 @@ int spg_block_sparse_attn(const int8_t *q8, const int8_t *k8, const uint8_t *v8,
   spg::Strides os;
   SPG_TRY(get_strides(fn, "out_strides", out_strides, H, N, D, &os));
   return check_launch(fn, spg::launch_block_sparse_attn(q8, k8, v8, out, os, out_dtype, lut, valid_block_num, pvthreshd,
-                                                        q_scale, k_scale, v_scale, B, H, Hkv, N, D, sm_scale,
+                                                        q_scale, k_scale, v_scale, B, H, Hkv, N, N_kv, D, sm_scale,
                                                         is_causal ? 1 : 0, pv_threshold_mode, pv_count, (hipStream_t)stream));
 }
 
@@ -187,10 +210,11 @@ int spg_v_tiles_f16(const void *v, const int64_t *v_strides, void *vt, int B, in
 int spg_block_sparse_attn_f16v(const int8_t *q8, const int8_t *k8, const void *vt, void *out, const int64_t *out_strides,
                                int out_dtype,
                                const int32_t *lut, const int32_t *valid_block_num, const float *pvthreshd,
-                               const float *q_scale, const float *k_scale, int B, int H, int Hkv, int N, int D,
+                               const float *q_scale, const float *k_scale, int B, int H, int Hkv, int N, int N_kv, int D,
                                float sm_scale, int is_causal, int pv_threshold_mode, int32_t *pv_count, void *stream) {
   const char *fn = "spg_block_sparse_attn_f16v";
   SPG_TRY(check_shape(fn, B, H, N, D));
+  SPG_TRY(check_shape(fn, B, Hkv > 0 ? Hkv : 1, N_kv, D));
   SPG_TRY(check_kv_heads(fn, H, Hkv));
   SPG_TRY(check_pv_mode(fn, pv_threshold_mode));
   SPG_TRY(check_dtype(fn, out_dtype));
@@ -199,7 +223,7 @@ int spg_block_sparse_attn_f16v(const int8_t *q8, const int8_t *k8, const void *v
   spg::Strides os;
   SPG_TRY(get_strides(fn, "out_strides", out_strides, H, N, D, &os));
   return check_launch(fn, spg::launch_block_sparse_attn(q8, k8, (const uint8_t *)vt, out, os, out_dtype, lut, valid_block_num,
-                                                        pvthreshd, q_scale, k_scale, nullptr, B, H, Hkv, N, D, sm_scale,
+                                                        pvthreshd, q_scale, k_scale, nullptr, B, H, Hkv, N, N_kv, D, sm_scale,
                                                         is_causal ? 1 : 0, pv_threshold_mode, pv_count, (hipStream_t)stream));
 }
 

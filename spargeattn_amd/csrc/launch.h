@@ -14,6 +14,11 @@ struct Strides {
 
 size_t km_mean_workspace_bytes(int B, int H, int N, int D);
 void launch_km_mean(const void *k, Strides ks, void *km, void *ws, int B, int H, int N, int D, int dtype, hipStream_t st);
+// size of the library-owned scratch array behind launch_km_mean_static (bytes); a shape whose
+// km_mean_workspace_bytes() exceeds it is refused by the caller
+#define SPG_KM_STATIC_SCRATCH_BYTES (8u << 20)
+size_t km_mean_static_capacity();
+hipError_t launch_km_mean_static(const void *k, Strides ks, void *km, int B, int H, int N, int D, int dtype, hipStream_t st);
 void launch_pool_sim_quant(const void *x, Strides xs, const void *km, void *pool, uint8_t *sim, int8_t *xq, float *scale,
                            const float *thr, int B, int H, int N, int D, int block, int dtype, hipStream_t st);
 int block_select_max_nk();
@@ -33,8 +38,9 @@ hipError_t launch_block_sparse_attn(const int8_t *q8, const int8_t *k8, const ui
                                     int out_dtype,
                                     const int32_t *lut, const int32_t *valid, const float *pvthreshd,
                                     const float *q_scale, const float *k_scale, const float *v_scale, int B, int H,
-                                    int Hkv, int N, int D, float sm_scale, int is_causal, int pv_mode,
+                                    int Hkv, int N, int Nk, int D, float sm_scale, int is_causal, int pv_mode,
                                     int32_t *pv_count, hipStream_t st);
+void launch_fp8_pack_selftest(const float *x, uint8_t *codes, int n, int saturate, hipStream_t st);
 
 hipError_t launch_dense_attn_f16(const void *q, const void *k, const void *v, void *out, int B, int H, int N, int D,
                                  float sm_scale, int is_causal, hipStream_t st);

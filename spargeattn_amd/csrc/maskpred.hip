@@ -17,6 +17,8 @@
 #include "common.h"
 #include "launch.h"
 
+#include <atomic>
+
 namespace spg {
 
 // =============================================================================================
@@ -913,6 +915,35 @@ void launch_km_mean(const void *k, Strides ks, void *km, void *ws, int B, int H,
   else         { if (dtype == 0) launch_km<128, 0>(k, ks, km, ws, B, H, N, st); else launch_km<128, 1>(k, ks, km, ws, B, H, N, st); }
 }
 
+// ---- K column mean without a caller-provided workspace ---------------------------------------------------------
+// The per-chunk partial sums go to a fixed array in device memory that the library owns (one copy per GPU, alive
+// until the process ends).  In host code the array's NAME is only a handle: its device address is asked for once per
+// device with hipGetSymbolAddress and that pointer is what the kernels receive.  Every call on a GPU shares the
+// array, so two calls that overlap in time on one GPU (different streams or threads) race; calls on one stream are
+// ordered.  Nothing needs clearing between calls: km_partial writes every partial sum km_final reads.
+static __device__ __align__(256) unsigned char km_static_scratch[SPG_KM_STATIC_SCRATCH_BYTES];
+
+size_t km_mean_static_capacity() { return SPG_KM_STATIC_SCRATCH_BYTES; }
+
+hipError_t launch_km_mean_static(const void *k, Strides ks, void *km, int B, int H, int N, int D, int dtype, hipStream_t st) {
+  constexpr int MAX_DEV = 64;
+  static std::atomic<void *> scratch_of_device[MAX_DEV];
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return e;
+  if (dev < 0 || dev >= MAX_DEV) return hipErrorInvalidDevice;
+  void *ptr = scratch_of_device[dev].load(std::memory_order_acquire);
+  if (ptr == nullptr) {
+    // first call on this device (the device is current): resolve this GPU's copy of the array
+    e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(km_static_scratch));
+    if (e != hipSuccess) return e;
+    if (ptr == nullptr) return hipErrorInvalidSymbol;
+    scratch_of_device[dev].store(ptr, std::memory_order_release);
+  }
+  launch_km_mean(k, ks, km, ptr, B, H, N, D, dtype, st);
+  return hipSuccess;
+}
+
 template <int BS, int D, int DT>
 static void launch_psq3(const void *x, Strides xs, const void *km, void *pool, uint8_t *sim, int8_t *xq, float *scale,
                         const float *thr, int B, int H, int N, hipStream_t st) {
@@ -944,6 +975,24 @@ void launch_pool_sim_quant(const void *x, Strides xs, const void *km, void *pool
 
 int block_select_max_nk() { return 8192; }
 
+// Kernels that need more than 48 KiB of dynamic LDS must be told so once (per device); the size granted last is
+// remembered per kernel and device, so the attribute call is not repeated on every launch.  gfx950 has 160 KiB of LDS
+// per workgroup; a request beyond it (including the kernel's static arrays, at most 4 KiB here) is refused up front.
+template <auto Kern>
+static hipError_t allow_dynamic_lds(size_t lds) {
+  if (lds + 4096 > 160 * 1024) return hipErrorInvalidConfiguration;
+  if (lds <= 48 * 1024) return hipSuccess;
+  static std::atomic<size_t> granted[32];
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return e;
+  const bool tracked = dev >= 0 && dev < 32;
+  if (tracked && granted[dev].load(std::memory_order_relaxed) >= lds) return hipSuccess;
+  e = hipFuncSetAttribute((const void *)Kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+  if (e == hipSuccess && tracked) granted[dev].store(lds, std::memory_order_relaxed);
+  return e;
+}
+
 void launch_div_selftest(unsigned long long *counts, int n_div, uint32_t seed, hipStream_t st) {
   div_selftest_kernel<<<(n_div + 255) / 256, 256, 0, st>>>(counts, n_div, seed);
 }
@@ -954,8 +1003,8 @@ static hipError_t launch_bs3(const void *pq, const uint8_t *sq, const void *pk, 
                              int H, int nq, int nk, int nkp, hipStream_t st) {
   const size_t lds = (size_t)R * D * 8 + (size_t)R * nkp * 4 + 12 * (size_t)nkp;
   auto kern = block_select_kernel<D, DT, R>;
-  if (lds > 48 * 1024) {
-    hipError_t e = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+  {
+    hipError_t e = allow_dynamic_lds<block_select_kernel<D, DT, R>>(lds);
     if (e != hipSuccess) return e;
   }
   kern<<<dim3((nq + R - 1) / R, B * H), 256, lds, st>>>((const uint16_t *)pq, sq, (const uint16_t *)pk, sk, topk, cdf,
@@ -974,8 +1023,8 @@ static hipError_t launch_bs2(const void *pq, const uint8_t *sq, const void *pk, 
     {                                                                                                           \
       const size_t lds = (size_t)R_ * D * 8 + (size_t)R_ * nkp * 4 + 16 * (size_t)nkp + 4 * 64 * 8;             \
       auto kern = block_select_wave_kernel<D, DT, R_, EPL_>;                                                    \
-      if (lds > 48 * 1024) {                                                                                    \
-        hipError_t e = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds); \
+      {                                                                                                         \
+        hipError_t e = allow_dynamic_lds<block_select_wave_kernel<D, DT, R_, EPL_>>(lds);                       \
         if (e != hipSuccess) return e;                                                                          \
       }                                                                                                         \
       kern<<<dim3((nq + R_ - 1) / R_, B * H), 256, lds, st>>>((const uint16_t *)pq, sq, (const uint16_t *)pk, sk, topk, \
@@ -991,7 +1040,9 @@ static hipError_t launch_bs2(const void *pq, const uint8_t *sq, const void *pk, 
   // rows per workgroup: reuse of the pooled-K reads against LDS footprint (scores are R*nkp floats)
   if (nkp <= 1024) return launch_bs3<D, DT, 8>(pq, sq, pk, sk, topk, cdf, causal, sink, lut, valid, bmap, B, H, nq, nk, nkp, st);
   if (nkp <= 4096) return launch_bs3<D, DT, 4>(pq, sq, pk, sk, topk, cdf, causal, sink, lut, valid, bmap, B, H, nq, nk, nkp, st);
-  return launch_bs3<D, DT, 2>(pq, sq, pk, sk, topk, cdf, causal, sink, lut, valid, bmap, B, H, nq, nk, nkp, st);
+  // nkp = 8192: one row per workgroup (D*8 + 16*nkp = 129 KiB; two rows would need 162 KiB, more than the 160 KiB a
+  // workgroup can have)
+  return launch_bs3<D, DT, 1>(pq, sq, pk, sk, topk, cdf, causal, sink, lut, valid, bmap, B, H, nq, nk, nkp, st);
 }
 
 hipError_t launch_block_select(const void *pq, const uint8_t *sq, const void *pk, const uint8_t *sk, const float *topk,
@@ -1011,8 +1062,8 @@ hipError_t launch_map_to_lut(const void *mask, int kind, int32_t *lut, int32_t *
 #define SPG_M2L(K_)                                                                                      \
   case K_: {                                                                                             \
     auto kern = map_to_lut_kernel<K_>;                                                                   \
-    if (lds > 48 * 1024) {                                                                               \
-      hipError_t e = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds); \
+    {                                                                                                    \
+      hipError_t e = allow_dynamic_lds<map_to_lut_kernel<K_>>(lds);                                      \
       if (e != hipSuccess) return e;                                                                     \
     }                                                                                                    \
     kern<<<grid, 256, lds, st>>>(mask, lut, valid, nq, nk, nkp);                                         \

@@ -19,7 +19,7 @@ def _declared():
 def test_header_declares_the_stages():
     names = _declared()
     for want in ("spg_km_mean", "spg_pool_sim_quant", "spg_block_select", "spg_map_to_lut", "spg_v_quant_fp8",
-                 "spg_block_sparse_attn", "spg_block_sparse_attn_f16v", "spg_v_tiles_f16", "spg_dense_attn_f16", "spg_selftest_division", "spg_last_error", "spg_version"):
+                 "spg_block_sparse_attn", "spg_block_sparse_attn_f16v", "spg_v_tiles_f16", "spg_dense_attn_f16", "spg_selftest_division", "spg_selftest_fp8_pack", "spg_last_error", "spg_version"):
         assert want in names
 
 
@@ -60,10 +60,14 @@ def test_argument_errors_are_reported_without_a_gpu():
     rc = lib.spg_v_quant_fp8(1, None, 1, 1, 1, 1, 128, 64, 7, None)
     assert rc == _lib.SPG_ERR_INVALID and b"dtype" in lib.spg_last_error()
     assert lib.spg_km_mean_workspace_bytes(1, 32, 32768, 128) > 0
-    rc = lib.spg_block_sparse_attn(1, 1, 1, 1, None, 0, 1, 1, 1, 1, 1, 1, 1, 6, 4, 128, 64, 0.125, 0, 1, None, None)
+    rc = lib.spg_block_sparse_attn(1, 1, 1, 1, None, 0, 1, 1, 1, 1, 1, 1, 1, 6, 4, 128, 128, 64, 0.125, 0, 1, None, None)
     assert rc == _lib.SPG_ERR_INVALID and b"must be divisible by num_kv_heads" in lib.spg_last_error()
-    rc = lib.spg_block_sparse_attn(1, 1, 1, 1, None, 0, 1, 1, 1, 1, 1, 1, 1, 4, 4, 128, 64, 0.125, 0, 3, None, None)
+    rc = lib.spg_block_sparse_attn(1, 1, 1, 1, None, 0, 1, 1, 1, 1, 1, 1, 1, 4, 4, 128, 128, 64, 0.125, 0, 3, None, None)
     assert rc == _lib.SPG_ERR_INVALID and b"pv_threshold_mode" in lib.spg_last_error()
+    rc = lib.spg_block_sparse_attn(1, 1, 1, 1, None, 0, 1, 1, 1, 1, 1, 1, 1, 4, 4, 128, 0, 64, 0.125, 0, 1, None, None)
+    assert rc == _lib.SPG_ERR_INVALID and b"must be positive" in lib.spg_last_error()        # kv_len
+    rc = lib.spg_selftest_fp8_pack(1, 1, 6, 1, None)
+    assert rc == _lib.SPG_ERR_INVALID and b"multiple of 4" in lib.spg_last_error()
     # strides: {batch, head, row} in elements, positive multiples of 8, row stride >= head_dim
     import ctypes
     bad = (ctypes.c_int64 * 3)(128 * 64, 64, 60)

@@ -313,3 +313,123 @@ def test_pv_threshold_modes_match_the_oracle(fp16v):
         counts[mode] = pvc.cpu().numpy().ravel().tolist()
     assert counts[_lib.PV_PER_BLOCK] == [nblk] * 4 * nqb == counts[_lib.PV_NONE]
     assert counts[_lib.PV_PER_WARP][1] < nblk and counts[_lib.PV_PER_WARP][:1] + counts[_lib.PV_PER_WARP][2:] == [nblk] * (4 * nqb - 1)
+
+
+def _int_case(n, nk_blocks, d, rng, r, a_blocks, hq=1):
+    """Hand-built quantised operands: small integer codes (diffuse rows) with per-block scales that put the exponent
+    multiplier a = sm_scale*log2(e)*q_scale*k_scale of each K block where the test wants it."""
+    nqb = (n + 127) // 128
+    q8 = rng.integers(-r, r + 1, size=(1, hq, n, d)).astype(np.int8)
+    k8 = rng.integers(-r, r + 1, size=(1, 1, n, d)).astype(np.int8)
+    lut = np.ones((1, hq, nqb, nk_blocks), np.int32); lut[..., 0] = 0
+    valid = np.full((1, hq, nqb), nk_blocks, np.int32)
+    c = np.float32(d ** -0.5) * np.float32(1.44269504)
+    qs = np.full((1, hq, nqb), 0.5, np.float32)
+    ks = (np.asarray(a_blocks, np.float32) / (c * np.float32(0.5))).reshape(1, 1, nk_blocks).astype(np.float32)
+    return q8, k8, lut, valid, qs, ks
+
+
+@pytest.mark.parametrize("fp16v", [False, True])
+@pytest.mark.parametrize("d,a_max", [(64, 2e-3), (128, 2e-2), (64, 0.1), (128, 0.5), (64, 2.25), (128, 9.0)])
+def test_large_exponent_multiplier_blocks(d, a_max, fp16v):
+    """Scores whose exponent multiplier a is far above what N(0,1) inputs give (large |q||k| or a large softmax scale):
+    the bias of the integer accumulators must leave the exponent without a rounding error that grows with a, and the
+    row maximum's probability must stay inside e4m3.  Blocks with small and large a alternate inside every row."""
+    nblk = 8
+    n = 64 * nblk
+    rng = np.random.default_rng(int(a_max * 1000) + d)
+    # codes in [-r, r]: std of a score ~ r^2/1.5 * sqrt(d); keep a*std around 2 so that rows stay diffuse
+    r = max(1, int(round((3.0 / (a_max * d ** 0.5)) ** 0.5)))
+    a_blocks = a_max * np.array([1.0, 1e-3, 0.5, 0.03, 1.0, 0.25, 1e-4, 0.7])
+    q8, k8, lut, valid, qs, ks = _int_case(n, nblk, d, rng, r, a_blocks)
+    thr = np.array([50.0], np.float32)
+    dev = lambda a: torch.from_numpy(a).cuda()
+    out = torch.zeros((1, 1, n, d), dtype=torch.float16, device="cuda")
+    if fp16v:
+        v = rng.standard_normal((1, 1, n, d)).astype(np.float16)
+        ref, _ = oat.block_sparse_attention(q8, k8, v.astype(np.float32), lut, valid, thr, qs, ks, None, d ** -0.5, "fp16", pv="f16")
+        _lib.block_sparse_attn_f16v(dev(q8), dev(k8), _lib.v_tiles_f16_swizzled(dev(v)), out, dev(lut), dev(valid), dev(thr),
+                                    dev(qs), dev(ks), d ** -0.5)
+    else:
+        vor = rng.integers(0, 120, size=(1, 1, n, d)).astype(np.uint8)
+        vs = np.ones((1, 1, d), np.float32)
+        ref, _ = oat.block_sparse_attention(q8, k8, vor, lut, valid, thr, qs, ks, vs, d ** -0.5, "fp16")
+        _lib.block_sparse_attn(dev(q8), dev(k8), _lib.v8_natural_to_tiles(dev(vor)), out, dev(lut), dev(valid), dev(thr),
+                               dev(qs), dev(ks), dev(vs), d ** -0.5)
+    assert torch.isfinite(out.float()).all()
+    met = _check_out(out, ref)
+    # the kernel follows the oracle far more closely than the operator tolerance: an exponent error of 0.75 a (what one
+    # rounding of the bias term costs at large a) would show here
+    assert met["L1"] <= 2e-3, met
+
+
+@pytest.mark.parametrize("mag,scale", [(30.0, None), (100.0, None), (300.0, None), (1.0, 8.0)])
+@pytest.mark.parametrize("D,dtype", [(64, torch.float16), (128, torch.bfloat16)])
+@pytest.mark.parametrize("sage1", [False, True])
+def test_operator_with_large_magnitude_inputs(mag, scale, D, dtype, sage1):
+    """Q and K scaled far beyond N(0,1), or a large explicit softmax scale: finite output within tolerance of the oracle."""
+    B, H, N = 1, 2, 512
+    q = rand_T((B, H, N, D), dtype, 80, scale=mag)
+    k = rand_T((B, H, N, D), dtype, 81, scale=mag, shift=0.4 * mag)
+    v = rand_T((B, H, N, D), dtype, 82)
+    if sage1:
+        res = oapi.spas_sage_attn_meansim_topk(to_np(q), to_np(k), to_np(v), tag_of(dtype), topk=0.75, scale=scale)
+        o = sa.spas_sage_attn_meansim_topk_cuda(q, k, v, topk=0.75, scale=scale)
+    else:
+        res = oapi.spas_sage2_attn_meansim_topk(to_np(q), to_np(k), to_np(v), tag_of(dtype), topk=0.75, scale=scale)
+        o = sa.spas_sage2_attn_meansim_topk_cuda(q, k, v, topk=0.75, scale=scale)
+    assert torch.isfinite(o.float()).all()
+    _check_out(o, res["out"])
+
+
+def test_fp8_pack_saturates_like_the_reference():
+    """The e4m3 pack of the attention kernel: round to nearest even below 448, +-448 beyond (cvt.rn.satfinite,
+    csrc/numeric_conversion.cuh:48-63), NaN stays NaN."""
+    from oracle import rounding as R
+    g = torch.Generator().manual_seed(9)
+    x = torch.cat([torch.tensor([0.0, 448.0, 449.0, 455.9, 463.9, 464.0, 464.1, 480.0, 1e3, 1e6, 3e38, float("inf"),
+                                 -449.0, -1e6, -float("inf"), 2.0 ** -9, 2.0 ** -10, 3 * 2.0 ** -11]),
+                   torch.rand(4096, generator=g) * 1000.0, torch.exp2(torch.rand(4096, generator=g) * 30 - 12),
+                   -torch.exp2(torch.rand(1022, generator=g) * 30 - 12)]).float()
+    assert x.numel() % 4 == 0
+    got = _lib.selftest_fp8_pack(x.cuda()).cpu().numpy()
+    want = R.f32_to_e4m3fn(x.numpy())
+    assert np.array_equal(got, want), [(float(a), hex(b), hex(c)) for a, b, c in zip(x, got, want) if b != c][:10]
+    nan = _lib.selftest_fp8_pack(torch.full((4,), float("nan"), device="cuda")).cpu().numpy()
+    assert np.all((nan & 0x7f) == 0x7f)
+
+
+def test_query_and_key_lengths_differ():
+    """qo_len != kv_len (csrc/qattn/qk_int_sv_f8_cuda_sm89.cu:256-300): a LUT of ceil(Nq/128) x ceil(Nk/64) blocks,
+    the last K block partial."""
+    B, H, D, dtype = 1, 2, 64, torch.float16
+    for Nq, Nk in ((384, 1000), (640, 200)):
+        q = rand_T((B, H, Nq, D), dtype, 90)
+        k = rand_T((B, H, Nk, D), dtype, 91, shift=0.3)
+        v = rand_T((B, H, Nk, D), dtype, 92)
+        res = oapi.spas_sage2_attn_meansim_topk(to_np(q), to_np(k), to_np(v), tag_of(dtype), topk=0.6)
+        o, sp = sa.spas_sage2_attn_meansim_topk_cuda(q, k, v, topk=0.6, return_sparsity=True)
+        assert o.shape == q.shape and abs(sp - res["sparsity"]) < 1e-6
+        _check_out(o, res["out"])
+        nq, nk = (Nq + 127) // 128, (Nk + 63) // 64
+        g = torch.Generator().manual_seed(6)
+        mask = (torch.rand((B, H, nq, nk), generator=g) < 0.6).to(torch.int32)
+        mask[..., nk - 1] = 1
+        res = oapi.block_sparse_sage2_attn(to_np(q), to_np(k), to_np(v), mask.numpy(), tag_of(dtype))
+        o = sa.block_sparse_sage2_attn_cuda(q, k, v, mask_id=mask.cuda())
+        _check_out(o, res["out"])
+    with pytest.raises(RuntimeError, match="inconsistent shapes"):
+        sa.spas_sage2_attn_meansim_topk_cuda(q, k, v[:, :, :128])
+
+
+def test_fp8_denominator_and_offset_construction():
+    """The kernel on the closed-form construction that separates "fp32 P in the denominator, e4m3(P) in the numerator,
+    offset 8.807" from "rounded P in the denominator" and from "no offset" (see tests/gpu_common.py)."""
+    from gpu_common import fp8_denominator_case
+    (q8, k8, v8, lut, valid, thr, qs, ks, vs, sm_scale), forms = fp8_denominator_case()
+    dev = lambda a: torch.from_numpy(a).cuda()
+    out = torch.zeros((1, 1, 128, 64), dtype=torch.float16, device="cuda")
+    _lib.block_sparse_attn(dev(q8), dev(k8), _lib.v8_natural_to_tiles(dev(v8)), out, dev(lut), dev(valid), dev(thr),
+                           dev(qs), dev(ks), dev(vs), sm_scale)
+    got = out.float().cpu().numpy()[0, 0]
+    assert np.all(np.abs(got - forms["reference"]) < 1.5e-3), (got[0, :4], forms)

@@ -154,3 +154,44 @@ def test_mask_operator_full_size_cfg2():
         cos, l1 = _cos_l1(o[b, h, r0:r0 + 128].float(), ref)
         print(f"cfg2 b{b} h{h} q-block {qb}: cos {cos:.6f} rel-L1 {l1:.4f}", flush=True)
         assert cos >= 0.995, (b, h, qb, cos, l1)                        # includes the INT8/FP8 quantisation error
+
+
+@pytest.mark.parametrize("name", ["cfg4", "cfg3"])
+def test_one_head_at_full_length_against_the_oracle(name):
+    """The headline configuration (and the D = 64 video one) at its REAL sequence length, one head: every stage the
+    oracle defines bit for bit (column mean, pooled blocks, similarity flags, INT8 codes and scales, block map, LUT,
+    FP8 codes and scales), the attention output at cos >= 0.999 / rel-L1 <= 1e-2."""
+    from oracle import api as oapi, attention as oat
+    from gpu_common import tag_of, to_np, bits_equal_T, v8_natural
+    cfg = W.CONFIGS[name]
+    q, k, v = W.make_qkv(cfg, device="cuda", shrink=dict(H=1))
+    B, H, N, D = q.shape
+    assert (H, N) == (1, cfg.N)
+    tag = tag_of(cfg.dtype)
+    print(f"{name}: oracle on {tuple(q.shape)} ...", flush=True)
+    res = oapi.spas_sage2_attn_meansim_topk(to_np(q), to_np(k), to_np(v), tag, is_causal=cfg.is_causal, topk=cfg.topk,
+                                            pvthreshd=cfg.pvthreshd)
+    print(f"{name}: oracle done, {int(res['valid'].sum())} blocks selected", flush=True)
+    km = _lib.km_mean(k)
+    assert bits_equal_T(km[:, :, 0], res["km"], cfg.dtype)
+    thr = torch.full((H,), -0.1, device="cuda")
+    pq, sq, q8, qs = _lib.pool_sim_quant(q, None, 128, thr)
+    pk, sk, k8, ks = _lib.pool_sim_quant(k, km, 64, thr)
+    assert bits_equal_T(pq, res["pool_q"], cfg.dtype) and bits_equal_T(pk, res["pool_k"], cfg.dtype)
+    assert np.array_equal(sq.cpu().numpy(), res["sim_q"]) and np.array_equal(sk.cpu().numpy(), res["sim_k"])
+    assert np.array_equal(q8.cpu().numpy(), res["q8"]) and np.array_equal(k8.cpu().numpy(), res["k8"])
+    assert np.array_equal(qs.cpu().numpy().view(np.uint32), res["q_scale"].view(np.uint32))
+    assert np.array_equal(ks.cpu().numpy().view(np.uint32), res["k_scale"].view(np.uint32))
+    topk = torch.full((H,), cfg.topk, device="cuda")
+    lut, valid, bmap = _lib.block_select(pq, sq, pk, sk, topk=topk, is_causal=cfg.is_causal, return_map=True)
+    assert np.array_equal(bmap.cpu().numpy(), res["map"])
+    assert np.array_equal(lut.cpu().numpy(), res["lut"]) and np.array_equal(valid.cpu().numpy(), res["valid"])
+    v8, vs = _lib.v_quant_fp8(v)
+    assert np.array_equal(v8_natural(v8, N), res["v8"][:, :, :N])
+    assert np.array_equal(vs.cpu().numpy().view(np.uint32), res["v_scale"].view(np.uint32))
+    o, sparsity = sa.spas_sage2_attn_meansim_topk_cuda(q, k, v, is_causal=cfg.is_causal, topk=cfg.topk,
+                                                       pvthreshd=cfg.pvthreshd, return_sparsity=True)
+    assert abs(sparsity - res["sparsity"]) < 1e-6
+    met = oat.precision_metric(to_np(o), res["out"])
+    print(f"{name}: full-length output vs oracle cos {met['Cossim']:.6f} rel-L1 {met['L1']:.2e}", flush=True)
+    assert met["Cossim"] >= 0.999 and met["L1"] <= 1e-2, met

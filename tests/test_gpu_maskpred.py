@@ -59,7 +59,8 @@ def _pools(B, H, nq, nk, D, dtype, seed):
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("nq,nk,D", [(8, 16, 64), (5, 9, 128), (139, 278, 64), (40, 300, 128), (3, 700, 128),
-                                     (5, 1500, 64), (3, 2100, 128)])   # last two: 32 columns per lane; the workgroup-level kernel
+                                     (5, 1500, 64), (3, 2100, 128),    # 32 columns per lane; the workgroup-level kernel
+                                     (2, 4100, 128), (2, 8192, 64)])   # one row per workgroup, the largest LDS footprint
 @pytest.mark.parametrize("mode", ["topk", "topk_causal", "cdf", "cdf_causal_sink"])
 def test_block_select(dtype, nq, nk, D, mode):
     tag = tag_of(dtype)

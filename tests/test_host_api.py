@@ -55,3 +55,55 @@ def test_workload_generators_shapes_and_determinism():
     i = torch.arange(8)
     assert m[:, :, i, 2 * i].all() and m[:, :, i, 2 * i + 1].all()
     assert 0.25 < m.float().mean() < 0.5
+
+
+def test_attention_wrapper_rejects_inconsistent_shapes_before_any_launch():
+    """The kernels index K, V, the LUT and the scales with ceil(kv_len/64): shapes that disagree must raise on the host."""
+    from spargeattn_amd import _lib
+    B, H, N, Nk, D = 1, 2, 256, 320, 64
+    nq, nk = 2, 5
+    q8 = torch.zeros((B, H, N, D), dtype=torch.int8)
+    k8 = torch.zeros((B, H, Nk, D), dtype=torch.int8)
+    v8 = torch.zeros((B, H, nk, D, 64), dtype=torch.uint8)
+    lut = torch.zeros((B, H, nq, nk), dtype=torch.int32)
+    valid = torch.zeros((B, H, nq), dtype=torch.int32)
+    qs, ks, vs = torch.ones((B, H, nq)), torch.ones((B, H, nk)), torch.ones((B, H, D))
+    assert _lib._check_attn_shapes(q8, k8, v8, lut, valid, qs, ks, vs) == (B, H, H, N, Nk, D)
+    with pytest.raises(RuntimeError, match="V tiles"):         # V quantised from a tensor as long as q, not as k
+        _lib._check_attn_shapes(q8, k8, torch.zeros((B, H, 4, D, 64), dtype=torch.uint8), lut, valid, qs, ks, vs)
+    with pytest.raises(RuntimeError, match="lut"):
+        _lib._check_attn_shapes(q8, k8, v8, torch.zeros((B, H, nq, 4), dtype=torch.int32), valid, qs, ks, vs)
+    with pytest.raises(RuntimeError, match="k_scale"):
+        _lib._check_attn_shapes(q8, k8, v8, lut, valid, qs, torch.ones((B, H, 4)), vs)
+    with pytest.raises(RuntimeError, match="does not match"):
+        _lib._check_attn_shapes(q8, torch.zeros((B, H, Nk, 128), dtype=torch.int8), v8, lut, valid, qs, ks, vs)
+    # the operator: k and v of different lengths
+    q = torch.zeros(1, 2, 256, 64, dtype=torch.float16)
+    with pytest.raises(RuntimeError, match="inconsistent shapes"):
+        sa.spas_sage2_attn_meansim_topk_cuda(q, q, q[:, :, :128])
+
+
+def test_broadcast_views_are_copied_not_passed_through():
+    """A stride of 0 (expand over heads) is not a layout the strided kernels read; the operator copies, as the
+    reference does with .contiguous() (core.py:113-117)."""
+    from spargeattn_amd import core
+    k = torch.zeros(1, 1, 256, 64, dtype=torch.float16).expand(1, 4, 256, 64)
+    assert k.stride(1) == 0
+    kc = core._rows_ok(k)
+    assert kc.is_contiguous() and kc.shape == k.shape
+    nhd = torch.zeros(1, 256, 4, 64, dtype=torch.bfloat16).transpose(1, 2)
+    assert core._rows_ok(nhd) is nhd                      # a plain NHD view is read in place
+
+
+def test_build_refuses_kernels_that_spill():
+    from spargeattn_amd import build
+    log = """attn.hip:1:1: remark: Function Name: kern_a [-Rpass-analysis=kernel-resource-usage]
+attn.hip:1:1: remark:     ScratchSize [bytes/lane]: 0 [-Rpass-analysis=kernel-resource-usage]
+attn.hip:1:1: remark:     VGPRs Spill: 0 [-Rpass-analysis=kernel-resource-usage]
+attn.hip:2:1: remark: Function Name: kern_b [-Rpass-analysis=kernel-resource-usage]
+attn.hip:2:1: remark:     ScratchSize [bytes/lane]: 24 [-Rpass-analysis=kernel-resource-usage]
+attn.hip:2:1: remark:     SGPRs Spill: 0 [-Rpass-analysis=kernel-resource-usage]
+attn.hip:2:1: remark:     VGPRs Spill: 6 [-Rpass-analysis=kernel-resource-usage]
+"""
+    bad = build._spill_report(log)
+    assert len(bad) == 2 and all(b.startswith("kern_b") for b in bad)

@@ -183,6 +183,21 @@ def test_f16v_denominator_uses_rounded_p():
     assert abs(got - rounded) < 4e-4 < abs(got - exact), (got, rounded, exact)
 
 
+def test_fp8_denominator_sums_unrounded_p_and_uses_the_offset():
+    """The two choices of the FP8 kernel that a tolerance test on random data cannot see (sm89.cuh:353-391,
+    attn_utils.cuh:28): the denominator sums the binary32 P while the numerator uses e4m3(P), and P carries the
+    2^8.807 factor that decides on which e4m3 grid it is rounded.  A construction whose closed form separates the
+    reference semantics from both alternatives by more than 0.04."""
+    from gpu_common import fp8_denominator_case
+    args, forms = fp8_denominator_case()
+    out, written, pvc = at.block_sparse_attention(*args[:9], args[9], "fp16", return_pv_count=True)
+    assert pvc[0, 0, 0] == 4
+    got = float(out[0, 0, 7, 3])
+    assert abs(got - forms["reference"]) < 1.5e-3, (got, forms)
+    assert abs(got - forms["rounded_denominator"]) > 0.03 and abs(got - forms["no_offset"]) > 0.03, (got, forms)
+    assert np.all(np.abs(out[0, 0] - got) < 1e-6)           # every row and channel alike
+
+
 def test_gqa_equals_mha_with_repeated_kv_heads():
     """Grouped-query attention: query head h reads K/V head h // (H / Hkv) (sm89.cuh:118).  With K/V heads repeated
     the multi-head path must give the identical result (quantisation is per K/V head, so nothing else changes)."""
