@@ -161,8 +161,10 @@ int spg_selftest_division(unsigned long long *counts, int n_divisors, unsigned i
 
 /* ---- self test (no counterpart in the reference): the fp32 -> e4m3 pack of the probabilities.
  * x (n,) float32 device, n a multiple of 4 -> codes (n,) uint8.  saturate != 0: exactly what spg_block_sparse_attn does
- * (round to nearest even, |x| > 448 clamps to +-448 like cvt.rn.satfinite.e4m3x2.f32, csrc/numeric_conversion.cuh:48-63);
- * saturate == 0: the bare v_cvt_pk_fp8_f32 instruction, for documentation of what the hardware does without the clamp. */
+ * (round to nearest even, finite |x| > 448 clamps to +-448 like cvt.rn.satfinite.e4m3x2.f32,
+ * csrc/numeric_conversion.cuh:48-63; NaN and +-inf give NaN - the reference maps +-inf to +-448, a case the kernel
+ * cannot reach because P = 2^x with x <= 8.807);
+ * saturate == 0: the bare v_cvt_pk_fp8_f32 instruction (NaN for |x| > 464), for documentation of the hardware. */
 int spg_selftest_fp8_pack(const float *x, uint8_t *codes, int n, int saturate, void *stream);
 
 #ifdef __cplusplus

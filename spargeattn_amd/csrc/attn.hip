@@ -76,7 +76,7 @@ __device__ __forceinline__ void lds_wait2(v4i &a, v4i &b) { asm volatile("s_wait
 __device__ __forceinline__ void lds_wait_acc(v16i &a, v16i &b) { asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(a), "+v"(b)); }
 
 // e4m3 pack of the probabilities.  v_cvt_pk_fp8_f32 returns NaN (0x7f) for |x| > 464 unless MODE.FP16_OVFL is set, in
-// which case it clamps to +-448 like the reference's cvt.rn.satfinite.e4m3x2.f32 (csrc/numeric_conversion.cuh:48-63);
+// which case finite values clamp to +-448 like the reference's cvt.rn.satfinite.e4m3x2.f32 (csrc/numeric_conversion.cuh:48-63);
 // the bit is set once per wavefront, costs nothing per element and affects no other instruction this kernel depends on
 // (the fp16 epilogue conversion cannot overflow: |O / d| <= max |V|).
 __device__ __forceinline__ void fp8_saturation_on() {

