@@ -29,18 +29,19 @@ SOURCES = {
 }
 # Translation units whose kernels read LDS through inline asm into registers the compiler believes are already
 # written: a spill or a scratch copy between such a read and its wait would store stale data, so the build fails
-# when any kernel of these files uses scratch memory or spills a register.
+# when any kernel of these files uses scratch memory or spills a vector register.  (Scalar registers parked in the
+# lanes of a vector register - "SGPRs Spill" - never touch memory or the registers those reads write, and are allowed.)
 NO_SPILL = {"attn.hip", "dense.hip"}
 RESOURCE_REMARKS = "-Rpass-analysis=kernel-resource-usage"
 
 
 def _spill_report(stderr):
-    """Kernel names of a -Rpass-analysis=kernel-resource-usage log that use scratch or spill registers."""
+    """Kernel names of a -Rpass-analysis=kernel-resource-usage log that use scratch or spill vector registers."""
     bad, name = [], None
     for line in stderr.splitlines():
         if "Function Name:" in line:
             name = line.split("Function Name:")[1].split("[")[0].strip()
-        for key in ("ScratchSize [bytes/lane]:", "SGPRs Spill:", "VGPRs Spill:"):
+        for key in ("ScratchSize [bytes/lane]:", "VGPRs Spill:"):
             if key in line:
                 value = line.split(key)[1].split("[")[0].strip()
                 if value != "0":

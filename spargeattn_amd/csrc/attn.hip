@@ -28,6 +28,8 @@
 #include "common.h"
 #include "launch.h"
 
+#include <type_traits>
+
 namespace spg {
 
 typedef int v4i __attribute__((ext_vector_type(4)));
@@ -38,8 +40,8 @@ typedef float v16f __attribute__((ext_vector_type(16)));
 
 #define SPG_NEG_BIG (-5000000.0f)   // csrc/qattn/attn_utils.cuh:350, qk_int_sv_f8_cuda_sm89.cuh:171
 #define SPG_FP8_OFFSET 8.807f       // csrc/qattn/attn_utils.cuh:28
-#define SPG_ACC_BIAS_BITS 0x4B400000 // 1.5 * 2^23 as an int32 and ...
-#define SPG_ACC_BIAS 12582912.0f     // ... as a float: floats in [2^23, 2^24) are the integers, one per bit pattern
+#define SPG_ACC_C_BITS 0x3E22F983    // the float 1/(2 pi), an inline constant of the instruction set: initial accumulator
+#define SPG_ACC_SCALE 67108864.0f    // 2^26: one unit of the integer dot product is 2^-26 in the binade [1/8, 1/4)
 #define SPG_LOG2E 1.44269504088896340736f
 
 struct AttnParams {
@@ -73,7 +75,6 @@ __device__ __forceinline__ void lds_wait4(v4i &a, v4i &b, v4i &c, v4i &d) {
   asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(a), "+v"(b), "+v"(c), "+v"(d));
 }
 __device__ __forceinline__ void lds_wait2(v4i &a, v4i &b) { asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(a), "+v"(b)); }
-__device__ __forceinline__ void lds_wait_acc(v16i &a, v16i &b) { asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(a), "+v"(b)); }
 
 // e4m3 pack of the probabilities.  v_cvt_pk_fp8_f32 returns NaN (0x7f) for |x| > 464 unless MODE.FP16_OVFL is set, in
 // which case finite values clamp to +-448 like the reference's cvt.rn.satfinite.e4m3x2.f32 (csrc/numeric_conversion.cuh:48-63);
@@ -141,12 +142,10 @@ __global__ __launch_bounds__(256, PV16 ? 2 : 3) void block_sparse_attn_kernel(co
   // LDS: K ring [NBUF][TILE] | V^T ring [NBUF][TILE] | votes
   __shared__ __align__(1024) unsigned char smem[NBUF * (TILE + VTILE)];
   __shared__ int sVote[2][4];
-  __shared__ __align__(16) int sBias[4];
   unsigned char *const sKr = smem;
   unsigned char *const sVr = smem + NBUF * TILE;
   const uint32_t lds_k0 = (uint32_t)(size_t)(__attribute__((address_space(3))) unsigned char *)smem;   // LDS byte address
   const uint32_t lds_v0 = lds_k0 + NBUF * TILE;
-  const uint32_t lds_bias = (uint32_t)(size_t)(__attribute__((address_space(3))) int *)sBias;
 
   // ---- workgroup -> (batch*head, q block): one XCD per head at a time, heavy (late) rows first ----------
   const int w = blockIdx.x;
@@ -165,7 +164,6 @@ __global__ __launch_bounds__(256, PV16 ? 2 : 3) void block_sparse_attn_kernel(co
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);   // uniform: everything derived from it stays scalar
   const int N = p.N, Nk = p.Nk;
   const int q_row = qb * 128 + wave * 32 + r;
-  if (tid < 4) sBias[tid] = SPG_ACC_BIAS_BITS;   // visible after the barrier that precedes the loop
   if constexpr (!PV16) fp8_saturation_on();
 
   // ---- Q fragment: B operand of S^T = K.Q^T, resident for the whole loop -------------------------------
@@ -271,29 +269,23 @@ __global__ __launch_bounds__(256, PV16 ? 2 : 3) void block_sparse_attn_kernel(co
   if (nv > 1) SPG_LOAD_TILES(blk1, TILE);
   uint32_t bufoff = 0;                     // LDS ring offset of block it
 
-  // The accumulators start at the bit pattern of 1.5 * 2^23: with |dot| < 2^22 the sums stay inside one binade, so the
-  // int32 result read as a float is exactly 12582912 + dot and no int-to-float conversion is needed.  The pattern is
-  // fetched from LDS (one 16-byte broadcast read per four registers), which costs no vector-ALU slot.  Every read issued
-  // from inline asm is waited for inside the iteration that issued it: the compiler does not know that the destination
-  // registers are written later, so a read still in flight when the loop exits would land on registers it has reused.
-  v16i S0, S1;
-#define SPG_LOAD_BIAS()                                                                                                 \
-  {                                                                                                                     \
-    v4i t0, t1, t2, t3, u0, u1, u2, u3;                                                                                 \
-    asm volatile("ds_read_b128 %0, %8\n\tds_read_b128 %1, %8\n\tds_read_b128 %2, %8\n\tds_read_b128 %3, %8\n\t"        \
-                 "ds_read_b128 %4, %8\n\tds_read_b128 %5, %8\n\tds_read_b128 %6, %8\n\tds_read_b128 %7, %8"               \
-                 : "=&v"(t0), "=&v"(t1), "=&v"(t2), "=&v"(t3), "=&v"(u0), "=&v"(u1), "=&v"(u2), "=&v"(u3)               \
-                 : "v"(lds_bias)                                                                                        \
-                 : "memory");                                                                                           \
-    S0 = (v16i){t0[0], t0[1], t0[2], t0[3], t1[0], t1[1], t1[2], t1[3], t2[0], t2[1], t2[2], t2[3], t3[0], t3[1], t3[2], t3[3]}; \
-    S1 = (v16i){u0[0], u0[1], u0[2], u0[3], u1[0], u1[1], u1[2], u1[3], u2[0], u2[1], u2[2], u2[3], u3[0], u3[1], u3[2], u3[3]}; \
-  }
+  // The INT8 accumulators do not start at zero but at the bit pattern 0x3E22F983 - the float 1/(2 pi), which the
+  // instruction set offers as an INLINE CONSTANT, so the first product of each chain takes it as its C operand and no
+  // register has to be initialised.  Its mantissa field is 2 292 099 and |dot| <= 128 * 128 * 128 = 2 097 152, so
+  // the int32 sum stays inside the binade [1/8, 1/4): the accumulator READ AS A FLOAT is exactly
+  // 1/(2 pi) + dot * 2^-26, and the scores need no int-to-float conversion - the 2^26 goes into the multiplier and the
+  // constant into the additive term of the fma that feeds exp2.
+  const float acc_c = __builtin_bit_cast(float, (int)SPG_ACC_C_BITS);
   __builtin_amdgcn_s_waitcnt(0x0F70);     // vmcnt(0): Q fragment and the first tiles have arrived
   __syncthreads();
-#pragma unroll 1
-  for (int it = 0; it < nv; it++) {
+
+  // One K block.  TAIL = false: every block but the last two - PV-threshold test, no masks (sm89.cuh:283-391).
+  // TAIL = true: the last two blocks - token-causal and out-of-bound masks, no skip (sm89.cuh:467-648).  The two are
+  // separate loops so that the common one carries none of the tail's predicates.
+  auto step = [&](auto tail_tag, const int it) __attribute__((always_inline)) {
+    constexpr bool TAIL = decltype(tail_tag)::value;
     // ---- S^T = K . Q^T ---------------------------------------------------------------------------------
-    SPG_LOAD_BIAS();
+    v16i S0, S1;
     {
       // two groups of k-steps: the reads of the second group are in flight while the first group's MFMAs run
       constexpr int HK = KS / 2;
@@ -302,11 +294,16 @@ __global__ __launch_bounds__(256, PV16 ? 2 : 3) void block_sparse_attn_kernel(co
 #pragma unroll
       for (int ks = 0; ks < HK; ks++) lds_read_2x128<0, 16 * D>(a0[ks], a1[ks], kaddr + ((uint32_t)(32 * ks) ^ k_rd_x));
       if constexpr (HK == 2) lds_wait4(a0[0], a1[0], a0[1], a1[1]); else lds_wait2(a0[0], a1[0]);
-      lds_wait_acc(S0, S1);   // the accumulator pattern has arrived as well (same counter); ties S0/S1 to the wait
 #pragma unroll
       for (int ks = HK; ks < KS; ks++) lds_read_2x128<0, 16 * D>(a0[ks], a1[ks], kaddr + ((uint32_t)(32 * ks) ^ k_rd_x));
+      // the first product of each chain, with the inline constant as its C operand (the compiler would otherwise keep
+      // the constant in sixteen registers); the products that follow accumulate onto these and are ordinary builtins,
+      // which the other chain's product always separates from their predecessor
+      asm volatile("v_mfma_i32_32x32x32_i8 %0, %2, %4, 0.15915494\n\tv_mfma_i32_32x32x32_i8 %1, %3, %4, 0.15915494"
+                   : "=&v"(S0), "=&v"(S1)
+                   : "v"(a0[0]), "v"(a1[0]), "v"(qreg[0]));
 #pragma unroll
-      for (int ks = 0; ks < HK; ks++) {
+      for (int ks = 1; ks < HK; ks++) {
         S0 = __builtin_amdgcn_mfma_i32_32x32x32_i8(a0[ks], qreg[ks], S0, 0, 0, 0);
         S1 = __builtin_amdgcn_mfma_i32_32x32x32_i8(a1[ks], qreg[ks], S1, 0, 0, 0);
       }
@@ -322,42 +319,43 @@ __global__ __launch_bounds__(256, PV16 ? 2 : 3) void block_sparse_attn_kernel(co
     // LDS loads share one counter, so a scalar load issued at the top of the loop would be waited for together with the
     // K operands; from here its latency runs under the MFMAs and the max reduction.
     __builtin_amdgcn_sched_barrier(0);
-    const float ksc2 = kscale[blk2];
-    const int d4 = it + 4 < nv ? lutc[it + 4] : 0;
+    float ksc2 = 0.f;
+    int d4 = 0;
+    if constexpr (!TAIL) {
+      ksc2 = kscale[blk2];
+      d4 = it + 4 < nv ? lutc[it + 4] : 0;
+    }
     __builtin_amdgcn_sched_barrier(0);
     const float dq = qs * ksc;
-    const bool tail = it >= nv - 2;   // last two blocks: masks, no PV skip (sm89.cuh:467-648)
     // S0/S1 are never rewritten (no copies at the join of the two paths): slot e < 16 is S0[e], slot e >= 16 is S1[e - 16]
     const float a = c * dq;
-    // The accumulator bias leaves the exponent through ONE additive constant, -(12582912 a + m) (+ 8.807), whose rounding
-    // error is half an ulp of 12582912 a.  Below 2^14 that is at most 2^-11 in the exponent (3e-4 relative in P, and the
+    const float a26 = a * SPG_ACC_SCALE;           // multiplier of the accumulator read as a float (exact scaling)
+    // The constant 1/(2 pi) leaves the exponent through ONE additive term, -(1/(2 pi) a 2^26 + m) (+ 8.807), whose rounding
+    // error is half an ulp of 1.07e7 a.  Below 2^14 that is at most 2^-11 in the exponent (3e-4 relative in P, and the
     // row maximum's P stays below 448.2).  At or above it (large |q| |k| or a large softmax scale; uniform for the
     // workgroup) the scores are first taken relative to the lane's own maximum - an exact subtraction inside one binade -
     // so that no large constant is left to round: one more instruction per score, on such blocks only.
-    const bool precise = a * SPG_ACC_BIAS >= 16384.0f;
-    float fm, mloc = SPG_ACC_BIAS;
-    auto tail_limit = [&]() {
-      const int key0 = blk * 64 + 32 * hh;
-      int lim = 0x7fffffff;
-      if (p.is_causal) lim = q_row - key0;                       // key > query (attn_utils.cuh:334-361)
-      if (it == nv - 1) lim = min(lim, Nk - 1 - key0);            // key >= kv_len (attn_utils.cuh:363-389)
-      return lim;
-    };
-    if (!tail) {
+    const bool precise = a26 * acc_c >= 16384.0f;
+    float fm, mloc = acc_c;
+    int lim = 0x7fffffff;
+    if constexpr (!TAIL) {
       int imax = S0[0];
 #pragma unroll
       for (int e = 1; e < 16; e++) imax = max(imax, S0[e]);
 #pragma unroll
       for (int e = 0; e < 16; e++) imax = max(imax, S1[e]);
-      fm = (float)(imax - SPG_ACC_BIAS_BITS) * a;
-      mloc = __builtin_bit_cast(float, imax);   // 12582912 + the largest of this lane's 32 dot products
+      fm = (float)(imax - SPG_ACC_C_BITS) * a;
+      mloc = __builtin_bit_cast(float, imax);   // 1/(2 pi) + 2^-26 * the largest of this lane's 32 dot products
     } else {
       // slot e of this lane is key 64*blk + 32*hh + e; keys beyond `lim` are masked
-      const int lim = tail_limit();
+      const int key0 = blk * 64 + 32 * hh;
+      if (p.is_causal) lim = q_row - key0;                       // key > query (attn_utils.cuh:334-361)
+      if (it == nv - 1) lim = min(lim, Nk - 1 - key0);           // key >= kv_len (attn_utils.cuh:363-389)
       fm = SPG_NEG_BIG;
+      const float dq26 = dq * SPG_ACC_SCALE;
 #pragma unroll
       for (int e = 0; e < 32; e++) {
-        float v = (__builtin_bit_cast(float, e < 16 ? S0[e] : S1[e - 16]) - SPG_ACC_BIAS) * dq;
+        float v = (__builtin_bit_cast(float, e < 16 ? S0[e] : S1[e - 16]) - acc_c) * dq26;
         v = e > lim ? SPG_NEG_BIG : v;
         fm = fmaxf(fm, v);
       }
@@ -369,7 +367,7 @@ __global__ __launch_bounds__(256, PV16 ? 2 : 3) void block_sparse_attn_kernel(co
     const float osc = __builtin_amdgcn_exp2f(m - m_new);
     m = m_new;
     int vote = 1;
-    if (!tail) {
+    if constexpr (!TAIL) {
       // max over rows of (diff) + thr > 0  <=>  some row has diff + thr > 0 (fp32 addition is monotonic)
       vote = __any(diff + thr > 0.f);
       if (lane == 0) sVote[it & 1][wave] = vote;
@@ -377,14 +375,14 @@ __global__ __launch_bounds__(256, PV16 ? 2 : 3) void block_sparse_attn_kernel(co
     __builtin_amdgcn_s_waitcnt(0x0F70);   // this wave's share of block it+1's tiles has landed in LDS
     __syncthreads();   // block it+1's tiles are complete; the votes are visible; ring slot of block it-1 is free
     bool compute = true;
-    if (!tail) {       // workgroup-uniform in the per-block mode (sm89.cuh:318-353), wavefront-uniform otherwise
+    if constexpr (!TAIL) {   // workgroup-uniform in the per-block mode (sm89.cuh:318-353), wavefront-uniform otherwise
       compute = p.pv_mode == 0 || vote != 0;
       // per-block mode: a wavefront whose own vote is set knows the OR already; only one that voted "skip" has to read
       // what the others wrote (an LDS round trip that the common case does without)
       if (p.pv_mode == 1 && !compute)
         compute = (sVote[it & 1][0] | sVote[it & 1][1] | sVote[it & 1][2] | sVote[it & 1][3]) != 0;
     }
-    if (it + 2 < nv) {
+    if (!TAIL || it + 2 < nv) {
       const uint32_t b2 = bufoff == 0 ? 2 * TILE : bufoff - TILE;   // slot (it+2) % 3
       SPG_LOAD_TILES(blk2, b2);
     }
@@ -400,20 +398,20 @@ __global__ __launch_bounds__(256, PV16 ? 2 : 3) void block_sparse_attn_kernel(co
       const float neg0 = PV16 ? -m : -m + SPG_FP8_OFFSET;
       float ps = 0.f;
       float x[32];
-      if (!tail) {
+      if constexpr (!TAIL) {
         // three passes kept apart for the scheduler: a multiply-add feeding the exponential of the same element directly,
         // and the exponential feeding the running sum, would issue as one long chain of dependent instructions
         if (!precise) {
-          const float neg = __builtin_fmaf(-SPG_ACC_BIAS, a, neg0);   // takes the accumulator bias out: one rounding per row
+          const float neg = __builtin_fmaf(-acc_c, a26, neg0);   // takes the accumulator constant out: one rounding per row
 #pragma unroll
-          for (int e = 0; e < 32; e++) x[e] = __builtin_fmaf(__builtin_bit_cast(float, e < 16 ? S0[e] : S1[e - 16]), a, neg);
+          for (int e = 0; e < 32; e++) x[e] = __builtin_fmaf(__builtin_bit_cast(float, e < 16 ? S0[e] : S1[e - 16]), a26, neg);
         } else {
           // (S - S_max,lane) a + (S_max,lane a - m + offset): what the reference's fma(S, a, -m + offset) computes
           // (attn_utils.cuh:391-415), with the rounding of m as the only error
-          const float c0 = __builtin_fmaf(mloc - SPG_ACC_BIAS, a, neg0);
+          const float c0 = __builtin_fmaf(mloc - acc_c, a26, neg0);
 #pragma unroll
           for (int e = 0; e < 32; e++)
-            x[e] = __builtin_fmaf(__builtin_bit_cast(float, e < 16 ? S0[e] : S1[e - 16]) - mloc, a, c0);
+            x[e] = __builtin_fmaf(__builtin_bit_cast(float, e < 16 ? S0[e] : S1[e - 16]) - mloc, a26, c0);
         }
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
@@ -424,12 +422,12 @@ __global__ __launch_bounds__(256, PV16 ? 2 : 3) void block_sparse_attn_kernel(co
           for (int e = 0; e < 32; e++) ps += x[e];
         }
       } else {
-        const int lim = tail_limit();
         const float masked = __builtin_fmaf(SPG_NEG_BIG, c, neg0);   // what the sentinel score turns into
+        const float dq26 = dq * SPG_ACC_SCALE;
 #pragma unroll
         for (int e = 0; e < 32; e++) {
           // de-quantised score first, then the softmax scale, as the reference's masked branch does (sm89.cuh:467-648)
-          const float sv = (__builtin_bit_cast(float, e < 16 ? S0[e] : S1[e - 16]) - SPG_ACC_BIAS) * dq;
+          const float sv = (__builtin_bit_cast(float, e < 16 ? S0[e] : S1[e - 16]) - acc_c) * dq26;
           const float t = __builtin_fmaf(sv, c, neg0);
           x[e] = __builtin_amdgcn_exp2f(e > lim ? masked : t);
           if constexpr (!PV16) ps += x[e];
@@ -526,9 +524,15 @@ __global__ __launch_bounds__(256, PV16 ? 2 : 3) void block_sparse_attn_kernel(co
     blk = blk1; blk1 = blk2; blk2 = blk2 + d3; d3 = d4;
     ksc = ksc1; ksc1 = ksc2;
     bufoff = bufoff == 2 * TILE ? 0 : bufoff + TILE;
+  };
+  {
+    int it = 0;
+#pragma unroll 1
+    for (; it < nv - 2; it++) step(std::false_type{}, it);
+#pragma unroll 1
+    for (; it < nv; it++) step(std::true_type{}, it);
   }
 #undef SPG_LOAD_TILES
-#undef SPG_LOAD_BIAS
 #undef SPG_LANE_OFFSETS
 
   // one count per wavefront of 32 query rows, the layout of the reference's PV_Count (sm89.cuh:650-659); the four
