@@ -89,12 +89,15 @@ int spg_pool_sim_quant(const void *x, const int64_t *x_strides, const void *km, 
  * triton_fill_causal_mask (304-316), triton_fill_block_map_kernel (282-302) and
  * triton_block_map_to_lut_kernel (54-87) with one kernel; the score matrix never reaches HBM.
  * Exactly one of topk / cdfthreshd ((H,) float32 device pointers) is non-NULL.
+ * pool_q (B,H,nq,D), sim_q (B,H,nq); pool_k (B,Hkv,nk,D), sim_k (B,Hkv,nk) with Hkv dividing H: query head h is scored
+ * against K head h / (H / Hkv).  Hkv = H is the reference's case; fewer K heads (grouped-query attention) is an
+ * extension - the reference's pooled-score matmul needs equal head counts (utils.py:388).
  * out: lut (B,H,nq,nk) int32 delta-encoded ascending block indices, zero tail;
  *      valid_block_num (B,H,nq) int32; block_map (B,H,nq,nk) uint8 0/1 or NULL. */
 int spg_block_select(const void *pool_q, const uint8_t *sim_q, const void *pool_k, const uint8_t *sim_k,
                      const float *topk, const float *cdfthreshd, int is_causal, int attention_sink,
                      int32_t *lut, int32_t *valid_block_num, uint8_t *block_map,
-                     int B, int H, int nq, int nk, int D, int dtype, void *stream);
+                     int B, int H, int Hkv, int nq, int nk, int D, int dtype, void *stream);
 
 /* ---- A8 alone: user block mask -> LUT  (block_map_lut_triton, spas_sage_attn/utils.py:76-87) ---- */
 int spg_map_to_lut(const void *mask, int mask_kind, int32_t *lut, int32_t *valid_block_num,

@@ -53,7 +53,9 @@ def spas_sage2_attn_meansim_topk(q, k, v, dtype, is_causal=False, scale=None, si
     res["km"] = km
     thr = hyperparameter(h, simthreshd1)
     rq = mp.pool_sim_quant(q, None, mp.BLKQ, thr, dtype)
-    rk = mp.pool_sim_quant(k, km, mp.BLKK, thr, dtype)
+    # grouped K/V heads (not in the reference, whose pooled-score matmul needs equal head counts): K is pooled once per
+    # K head with the similarity threshold of the first query head of its group
+    rk = mp.pool_sim_quant(k, km, mp.BLKK, thr[::h // k.shape[1]], dtype)
     res.update(pool_q=rq["pool"], sim_q=rq["sim"], q8=rq["q"], q_scale=rq["scale"],
                pool_k=rk["pool"], sim_k=rk["sim"], k8=rk["q"], k_scale=rk["scale"])
     fmap = mp.block_map(rq["pool"], rq["sim"], rk["pool"], rk["sim"], dtype, is_causal=is_causal,
@@ -82,9 +84,10 @@ def spas_sage_attn_meansim_topk(q, k, v, dtype, is_causal=False, scale=None, sim
                                        stop_after_mask=True)
     q = np.asarray(q, dtype=F32)
     b, h, n, d = q.shape
-    nk = (n + 63) // 64
-    v16 = np.zeros((b, h, nk * 64, d), dtype=F32)
-    v16[:, :, :n] = vq.to_fp16(v)
+    hkv, nkv = np.shape(v)[1], np.shape(v)[2]              # K/V may have fewer heads and another length than Q
+    nk = (nkv + 63) // 64
+    v16 = np.zeros((b, hkv, nk * 64, d), dtype=F32)
+    v16[:, :, :nkv] = vq.to_fp16(v)
     res["v16"] = v16
     sm_scale = (1.0 / d ** 0.5) if scale is None else scale
     out, written, pvc = at.block_sparse_attention(

@@ -256,10 +256,17 @@ def num_to_select_cdf(p, order, cdfthreshd, dtype):
 
 def block_map(pool_q, sim_q, pool_k, sim_k, dtype, is_causal=False, topk=None, cdfthreshd=None,
               attention_sink=False, return_probs=False):
-    """Steps 4-8: boolean block map (B,H,nq,nk) (utils.py:386-415)."""
+    """Steps 4-8: boolean block map (B,H,nq,nk) (utils.py:386-415).
+
+    pool_k / sim_k may carry fewer heads than pool_q (grouped K/V heads, an extension the reference's matmul at
+    utils.py:388 does not have): query head h then uses K head h // (H / Hkv), i.e. the K tensors repeated per group."""
     assert (topk is None) != (cdfthreshd is None), "Only one of cdfthreshd and topk can be set."
     b, h, nq, _ = pool_q.shape
     nk = pool_k.shape[2]
+    if pool_k.shape[1] != h:
+        assert h % pool_k.shape[1] == 0
+        pool_k = np.repeat(pool_k, h // pool_k.shape[1], axis=1)
+        sim_k = np.repeat(sim_k, h // sim_k.shape[1], axis=1)
     score = pooled_scores(pool_q, pool_k, dtype).astype(F32)
     score = np.where(sim_k[:, :, None, :], score, -np.inf)
     cm = causal_block_mask(nq, nk)

@@ -27,7 +27,7 @@ SIGNATURES = {
     "spg_km_mean": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp]),
     "spg_km_mean_static": (_i, [_vp, _vp, _vp, _i, _i, _i, _i, _i, _vp]),
     "spg_pool_sim_quant": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp]),
-    "spg_block_select": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp]),
+    "spg_block_select": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _vp]),
     "spg_map_to_lut": (_i, [_vp, _i, _vp, _vp, _i, _i, _i, _i, _vp]),
     "spg_v_quant_fp8": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp]),
     "spg_block_sparse_attn": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _f, _i, _i, _vp, _vp]),
@@ -110,8 +110,11 @@ def _st(t):
     return (ctypes.c_int64 * 3)(t.stride(0), t.stride(1), t.stride(2))
 
 
-def _stream():
-    return torch.cuda.current_stream().cuda_stream
+def _stream(stream=None):
+    """Raw HIP stream handle: torch's current stream, or the given torch stream.  Wrappers that take ``stream=``
+    allocate their outputs in the caller's (current) stream context and only LAUNCH on the given one, so the caching
+    allocator keeps treating the outputs as the caller's; the caller orders the two streams with events."""
+    return (torch.cuda.current_stream() if stream is None else stream).cuda_stream
 
 
 _MASK_KIND = {
@@ -135,7 +138,7 @@ def km_mean(k):
     return km
 
 
-def pool_sim_quant(x, km, block, simthreshd1=None, with_pool=True):
+def pool_sim_quant(x, km, block, simthreshd1=None, with_pool=True, stream=None):
     """Returns (pool, sim, x_int8, scale) - pool and sim are None when with_pool is False."""
     _dev_strided(x)
     _dev(km, simthreshd1)
@@ -148,7 +151,7 @@ def pool_sim_quant(x, km, block, simthreshd1=None, with_pool=True):
         pool = torch.empty((B, H, nb, D), dtype=x.dtype, device=x.device)
         sim = torch.empty((B, H, nb), dtype=torch.bool, device=x.device)
     _check(load().spg_pool_sim_quant(_p(x), _st(x), _p(km), _p(pool), _p(sim), _p(xq), _p(scale), _p(simthreshd1),
-                                     B, H, N, D, block, _dt(x), _stream()))
+                                     B, H, N, D, block, _dt(x), _stream(stream)))
     return pool, sim, xq, scale
 
 
@@ -156,13 +159,19 @@ def block_select(pool_q, sim_q, pool_k, sim_k, topk=None, cdfthreshd=None, is_ca
                  attention_sink=False, return_map=False):
     _dev(pool_q, sim_q, pool_k, sim_k, topk, cdfthreshd)
     B, H, nq, D = pool_q.shape
-    nk = pool_k.shape[2]
+    Hkv, nk = pool_k.shape[1], pool_k.shape[2]
+    if (pool_k.shape[0], pool_k.shape[3]) != (B, D) or tuple(sim_q.shape) != (B, H, nq) or tuple(sim_k.shape) != (B, Hkv, nk):
+        raise RuntimeError(f"pooled tensors disagree: pool_q {tuple(pool_q.shape)}, sim_q {tuple(sim_q.shape)}, "
+                           f"pool_k {tuple(pool_k.shape)}, sim_k {tuple(sim_k.shape)}")
+    for t in (topk, cdfthreshd):
+        if t is not None and t.numel() != H:
+            raise RuntimeError(f"per-head hyper-parameter has {t.numel()} entries, expected {H}")
     lut = torch.empty((B, H, nq, nk), dtype=torch.int32, device=pool_q.device)
     valid = torch.empty((B, H, nq), dtype=torch.int32, device=pool_q.device)
     bmap = torch.empty((B, H, nq, nk), dtype=torch.bool, device=pool_q.device) if return_map else None
     _check(load().spg_block_select(_p(pool_q), _p(sim_q), _p(pool_k), _p(sim_k), _p(topk), _p(cdfthreshd),
                                    int(bool(is_causal)), int(bool(attention_sink)), _p(lut), _p(valid), _p(bmap),
-                                   B, H, nq, nk, D, _dt(pool_q), _stream()))
+                                   B, H, Hkv, nq, nk, D, _dt(pool_q), _stream()))
     return lut, valid, bmap
 
 
@@ -177,14 +186,14 @@ def map_to_lut(block_map):
     return lut, valid
 
 
-def v_quant_fp8(v):
+def v_quant_fp8(v, stream=None):
     """v (B,H,N,D) fp16/bf16 -> (v8 uint8 codes in tile layout (B,H,nk,D,64), v_scale (B,H,D) float32)."""
     _dev_strided(v)
     B, H, N, D = v.shape
     nk = (N + 63) // 64
     v8 = torch.empty((B, H, nk, D, 64), dtype=torch.uint8, device=v.device)
     v_scale = torch.empty((B, H, D), dtype=torch.float32, device=v.device)
-    _check(load().spg_v_quant_fp8(_p(v), _st(v), _p(v8), _p(v_scale), B, H, N, D, _dt(v), _stream()))
+    _check(load().spg_v_quant_fp8(_p(v), _st(v), _p(v8), _p(v_scale), B, H, N, D, _dt(v), _stream(stream)))
     return v8, v_scale
 
 
@@ -252,13 +261,13 @@ def block_sparse_attn(q8, k8, v8, out, lut, valid, pvthreshd, q_scale, k_scale, 
     return pvc
 
 
-def v_tiles_f16_swizzled(v):
+def v_tiles_f16_swizzled(v, stream=None):
     """v (B,H,N,D) fp16/bf16 -> (B,H,nk,D,64) fp16 V^T tiles, chunk-swizzled, the operand of block_sparse_attn_f16v."""
     _dev_strided(v)
     B, H, N, D = v.shape
     nk = (N + 63) // 64
     vt = torch.empty((B, H, nk, D, 64), dtype=torch.float16, device=v.device)
-    _check(load().spg_v_tiles_f16(_p(v), _st(v), _p(vt), B, H, N, D, _dt(v), _stream()))
+    _check(load().spg_v_tiles_f16(_p(v), _st(v), _p(vt), B, H, N, D, _dt(v), _stream(stream)))
     return vt
 
 

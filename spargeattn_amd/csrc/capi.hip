@@ -121,10 +121,11 @@ int spg_pool_sim_quant(const void *x, const int64_t *x_strides, const void *km, 
 
 int spg_block_select(const void *pool_q, const uint8_t *sim_q, const void *pool_k, const uint8_t *sim_k,
                      const float *topk, const float *cdfthreshd, int is_causal, int attention_sink, int32_t *lut,
-                     int32_t *valid_block_num, uint8_t *block_map, int B, int H, int nq, int nk, int D, int dtype,
+                     int32_t *valid_block_num, uint8_t *block_map, int B, int H, int Hkv, int nq, int nk, int D, int dtype,
                      void *stream) {
   const char *fn = "spg_block_select";
   if (B <= 0 || H <= 0 || nq <= 0 || nk <= 0) return fail(SPG_ERR_INVALID, "%s: B, H, nq, nk must be positive", fn);
+  SPG_TRY(check_kv_heads(fn, H, Hkv));
   if (D != 64 && D != 128) return fail(SPG_ERR_UNSUPPORTED, "%s: head_dim must be 64 or 128 (got %d)", fn, D);
   SPG_TRY(check_dtype(fn, dtype));
   if ((topk == nullptr) == (cdfthreshd == nullptr))
@@ -134,8 +135,8 @@ int spg_block_select(const void *pool_q, const uint8_t *sim_q, const void *pool_
   SPG_NONNULL(fn, pool_q); SPG_NONNULL(fn, sim_q); SPG_NONNULL(fn, pool_k); SPG_NONNULL(fn, sim_k);
   SPG_NONNULL(fn, lut); SPG_NONNULL(fn, valid_block_num);
   return check_launch(fn, spg::launch_block_select(pool_q, sim_q, pool_k, sim_k, topk, cdfthreshd, is_causal ? 1 : 0,
-                                                   attention_sink ? 1 : 0, lut, valid_block_num, block_map, B, H, nq,
-                                                   nk, D, dtype, (hipStream_t)stream));
+                                                   attention_sink ? 1 : 0, lut, valid_block_num, block_map, B, H, Hkv,
+                                                   nq, nk, D, dtype, (hipStream_t)stream));
 }
 
 int spg_map_to_lut(const void *mask, int mask_kind, int32_t *lut, int32_t *valid_block_num, int B, int H, int nq,

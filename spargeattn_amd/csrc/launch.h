@@ -24,7 +24,7 @@ void launch_pool_sim_quant(const void *x, Strides xs, const void *km, void *pool
 int block_select_max_nk();
 hipError_t launch_block_select(const void *pq, const uint8_t *sq, const void *pk, const uint8_t *sk, const float *topk,
                                const float *cdf, int causal, int sink, int32_t *lut, int32_t *valid, uint8_t *bmap,
-                               int B, int H, int nq, int nk, int D, int dtype, hipStream_t st);
+                               int B, int H, int Hkv, int nq, int nk, int D, int dtype, hipStream_t st);
 void launch_div_selftest(unsigned long long *counts, int n_div, uint32_t seed, hipStream_t st);
 hipError_t launch_map_to_lut(const void *mask, int kind, int32_t *lut, int32_t *valid, int B, int H, int nq, int nk,
                              hipStream_t st);

@@ -396,8 +396,8 @@ template <int D, int DT, int R>
 __global__ __launch_bounds__(256) void block_select_kernel(
     const uint16_t *__restrict__ pool_q, const uint8_t *__restrict__ sim_q, const uint16_t *__restrict__ pool_k,
     const uint8_t *__restrict__ sim_k, const float *__restrict__ topk, const float *__restrict__ cdfthr, int is_causal,
-    int sink, int32_t *__restrict__ lut, int32_t *__restrict__ valid, uint8_t *__restrict__ bmap, int H, int nq, int nk,
-    int nkp) {
+    int sink, int32_t *__restrict__ lut, int32_t *__restrict__ valid, uint8_t *__restrict__ bmap, int H, int Hkv, int nq,
+    int nk, int nkp) {
   extern __shared__ __align__(16) unsigned char smem[];
   double *s_pq = (double *)smem;                                   // [R][D]
   float *s_scores = (float *)(smem + (size_t)R * D * 8);           // [R][nkp]
@@ -421,8 +421,10 @@ __global__ __launch_bounds__(256) void block_select_kernel(
   __syncthreads();
 
   const float sm_scale = (D == 64) ? 0.125f : 0.088388347648318447f;  // fp32(D^-0.5)
-  const uint16_t *pk_base = pool_k + (size_t)bh * nk * D;
-  const uint8_t *simk = sim_k + (size_t)bh * nk;
+  // grouped K/V heads: query head h is scored against the pooled blocks of K head h / (H / Hkv)
+  const int bhk = (bh / H) * Hkv + h / (H / Hkv);
+  const uint16_t *pk_base = pool_k + (size_t)bhk * nk * D;
+  const uint8_t *simk = sim_k + (size_t)bhk * nk;
 
   // ---- phase 1: scores.  Products of two 16-bit floats are exact in binary64, so fma == multiply-then-add. ----
   for (int j = tid; j < nk; j += 256) {
@@ -618,7 +620,7 @@ template <int D, int DT, int R, int EPL>
 __global__ __launch_bounds__(256) void block_select_wave_kernel(
     const uint16_t *__restrict__ pool_q, const uint8_t *__restrict__ sim_q, const uint16_t *__restrict__ pool_k,
     const uint8_t *__restrict__ sim_k, const float *__restrict__ topk, const float *__restrict__ cdfthr, int is_causal,
-    int sink, int32_t *__restrict__ lut, int32_t *__restrict__ valid, uint8_t *__restrict__ bmap, int H, int nq,
+    int sink, int32_t *__restrict__ lut, int32_t *__restrict__ valid, uint8_t *__restrict__ bmap, int H, int Hkv, int nq,
     int nk) {
   constexpr int NKP = 64 * EPL;
   extern __shared__ __align__(16) unsigned char smem[];
@@ -640,8 +642,10 @@ __global__ __launch_bounds__(256) void block_select_wave_kernel(
   __syncthreads();
 
   const float sm_scale = (D == 64) ? 0.125f : 0.088388347648318447f;  // fp32(D^-0.5)
-  const uint16_t *pk_base = pool_k + (size_t)bh * nk * D;
-  const uint8_t *simk = sim_k + (size_t)bh * nk;
+  // grouped K/V heads: query head h is scored against the pooled blocks of K head h / (H / Hkv)
+  const int bhk = (bh / H) * Hkv + h / (H / Hkv);
+  const uint16_t *pk_base = pool_k + (size_t)bhk * nk * D;
+  const uint8_t *simk = sim_k + (size_t)bhk * nk;
 
   // ---- phase 1: scores, binary64 accumulation in the fixed order d = 0..D-1 (products of 16-bit floats are exact) ----
   // columns at or beyond j_live are masked for every row of this workgroup: no arithmetic for them
@@ -1000,7 +1004,7 @@ void launch_div_selftest(unsigned long long *counts, int n_div, uint32_t seed, h
 template <int D, int DT, int R>
 static hipError_t launch_bs3(const void *pq, const uint8_t *sq, const void *pk, const uint8_t *sk, const float *topk,
                              const float *cdf, int causal, int sink, int32_t *lut, int32_t *valid, uint8_t *bmap, int B,
-                             int H, int nq, int nk, int nkp, hipStream_t st) {
+                             int H, int Hkv, int nq, int nk, int nkp, hipStream_t st) {
   const size_t lds = (size_t)R * D * 8 + (size_t)R * nkp * 4 + 12 * (size_t)nkp;
   auto kern = block_select_kernel<D, DT, R>;
   {
@@ -1008,14 +1012,14 @@ static hipError_t launch_bs3(const void *pq, const uint8_t *sq, const void *pk, 
     if (e != hipSuccess) return e;
   }
   kern<<<dim3((nq + R - 1) / R, B * H), 256, lds, st>>>((const uint16_t *)pq, sq, (const uint16_t *)pk, sk, topk, cdf,
-                                                        causal, sink, lut, valid, bmap, H, nq, nk, nkp);
+                                                        causal, sink, lut, valid, bmap, H, Hkv, nq, nk, nkp);
   return hipSuccess;
 }
 
 template <int D, int DT>
 static hipError_t launch_bs2(const void *pq, const uint8_t *sq, const void *pk, const uint8_t *sk, const float *topk,
                              const float *cdf, int causal, int sink, int32_t *lut, int32_t *valid, uint8_t *bmap, int B,
-                             int H, int nq, int nk, hipStream_t st) {
+                             int H, int Hkv, int nq, int nk, hipStream_t st) {
   const int nkp = next_pow2_ge(nk, 256);
   if (nkp <= 2048) {
     // a whole row fits the registers of one wavefront
@@ -1028,7 +1032,7 @@ static hipError_t launch_bs2(const void *pq, const uint8_t *sq, const void *pk, 
         if (e != hipSuccess) return e;                                                                          \
       }                                                                                                         \
       kern<<<dim3((nq + R_ - 1) / R_, B * H), 256, lds, st>>>((const uint16_t *)pq, sq, (const uint16_t *)pk, sk, topk, \
-                                                              cdf, causal, sink, lut, valid, bmap, H, nq, nk);  \
+                                                              cdf, causal, sink, lut, valid, bmap, H, Hkv, nq, nk); \
       return hipSuccess;                                                                                        \
     }
     if (nkp == 256) SPG_BSW(8, 4)
@@ -1038,17 +1042,17 @@ static hipError_t launch_bs2(const void *pq, const uint8_t *sq, const void *pk, 
 #undef SPG_BSW
   }
   // rows per workgroup: reuse of the pooled-K reads against LDS footprint (scores are R*nkp floats)
-  if (nkp <= 1024) return launch_bs3<D, DT, 8>(pq, sq, pk, sk, topk, cdf, causal, sink, lut, valid, bmap, B, H, nq, nk, nkp, st);
-  if (nkp <= 4096) return launch_bs3<D, DT, 4>(pq, sq, pk, sk, topk, cdf, causal, sink, lut, valid, bmap, B, H, nq, nk, nkp, st);
+  if (nkp <= 1024) return launch_bs3<D, DT, 8>(pq, sq, pk, sk, topk, cdf, causal, sink, lut, valid, bmap, B, H, Hkv, nq, nk, nkp, st);
+  if (nkp <= 4096) return launch_bs3<D, DT, 4>(pq, sq, pk, sk, topk, cdf, causal, sink, lut, valid, bmap, B, H, Hkv, nq, nk, nkp, st);
   // nkp = 8192: one row per workgroup (D*8 + 16*nkp = 129 KiB; two rows would need 162 KiB, more than the 160 KiB a
   // workgroup can have)
-  return launch_bs3<D, DT, 1>(pq, sq, pk, sk, topk, cdf, causal, sink, lut, valid, bmap, B, H, nq, nk, nkp, st);
+  return launch_bs3<D, DT, 1>(pq, sq, pk, sk, topk, cdf, causal, sink, lut, valid, bmap, B, H, Hkv, nq, nk, nkp, st);
 }
 
 hipError_t launch_block_select(const void *pq, const uint8_t *sq, const void *pk, const uint8_t *sk, const float *topk,
                                const float *cdf, int causal, int sink, int32_t *lut, int32_t *valid, uint8_t *bmap,
-                               int B, int H, int nq, int nk, int D, int dtype, hipStream_t st) {
-#define SPG_BS(D_, DT_) return launch_bs2<D_, DT_>(pq, sq, pk, sk, topk, cdf, causal, sink, lut, valid, bmap, B, H, nq, nk, st)
+                               int B, int H, int Hkv, int nq, int nk, int D, int dtype, hipStream_t st) {
+#define SPG_BS(D_, DT_) return launch_bs2<D_, DT_>(pq, sq, pk, sk, topk, cdf, causal, sink, lut, valid, bmap, B, H, Hkv, nq, nk, st)
   if (D == 64) { if (dtype == 0) SPG_BS(64, 0); else SPG_BS(64, 1); }
   else         { if (dtype == 0) SPG_BS(128, 0); else SPG_BS(128, 1); }
 #undef SPG_BS

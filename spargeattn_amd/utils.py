@@ -93,18 +93,21 @@ def get_block_map_meansim_fuse_quant(q, k, km=None, is_causal=False, BLKQ=128, B
     assert (cdfthreshd is None and topk is not None) \
         or (cdfthreshd is not None and topk is None), "Only one of cdfthreshd and topk can be set."
     _check_blocks(BLKQ, BLKK)
-    H = q.size(1)
-    if k.size(1) != H:
-        # the reference's pooled-score matmul fails on mismatching head counts (utils.py:388)
-        raise RuntimeError(f"mask prediction needs as many K heads as Q heads (got {k.size(1)} and {H}); "
-                           "grouped-query attention is supported by block_sparse_sage2_attn_cuda only")
+    H, Hkv = q.size(1), k.size(1)
+    if Hkv <= 0 or H % Hkv != 0:
+        # the message of the reference's kernel entry (qk_int_sv_f8_cuda_sm89.cu:310-314)
+        raise ValueError(f"num_qo_heads ({H}) must be divisible by num_kv_heads ({Hkv})")
     simthreshd1 = hyperparameter_check(simthreshd1, H, q.device)
     if cdfthreshd is not None:
         cdfthreshd = hyperparameter_check(cdfthreshd, H, q.device)
     if topk is not None:
         topk = hyperparameter_check(topk, H, q.device)
     pool_q, sim_q, q_int8, q_scale = _lib.pool_sim_quant(q, None, BLKQ, simthreshd1)
-    pool_k, sim_k, k_int8, k_scale = _lib.pool_sim_quant(k, km, BLKK, simthreshd1)
+    # Grouped K/V heads (an extension: the reference's pooled-score matmul needs Hkv == H, utils.py:388).  K is pooled and
+    # quantised once per K head; its similarity flags use the threshold of the FIRST query head of the group; every query
+    # head of the group is scored against those pooled blocks with its own topk / cdfthreshd.
+    simthreshd1_k = simthreshd1 if Hkv == H else simthreshd1[::H // Hkv].contiguous()
+    pool_k, sim_k, k_int8, k_scale = _lib.pool_sim_quant(k, km, BLKK, simthreshd1_k)
     lut, valid, bmap = _lib.block_select(pool_q, sim_q, pool_k, sim_k, topk=topk, cdfthreshd=cdfthreshd,
                                          is_causal=is_causal, attention_sink=attention_sink,
                                          return_map=not return_lut)

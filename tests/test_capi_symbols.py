@@ -53,8 +53,10 @@ def test_argument_errors_are_reported_without_a_gpu():
     lib = _lib.load()
     rc = lib.spg_km_mean(None, None, None, None, 1, 1, 128, 96, 0, None)
     assert rc == _lib.SPG_ERR_UNSUPPORTED and b"head_dim" in lib.spg_last_error()
-    rc = lib.spg_block_select(1, 1, 1, 1, None, None, 0, 0, 1, 1, None, 1, 1, 1, 2, 64, 0, None)
+    rc = lib.spg_block_select(1, 1, 1, 1, None, None, 0, 0, 1, 1, None, 1, 1, 1, 1, 2, 64, 0, None)
     assert rc == _lib.SPG_ERR_INVALID and b"Only one of cdfthreshd and topk" in lib.spg_last_error()
+    rc = lib.spg_block_select(1, 1, 1, 1, 1, None, 0, 0, 1, 1, None, 1, 6, 4, 1, 2, 64, 0, None)
+    assert rc == _lib.SPG_ERR_INVALID and b"must be divisible by num_kv_heads" in lib.spg_last_error()
     rc = lib.spg_pool_sim_quant(None, None, None, None, None, None, None, None, 1, 1, 128, 64, 128, 1, None)
     assert rc == _lib.SPG_ERR_INVALID and b"NULL" in lib.spg_last_error()
     rc = lib.spg_v_quant_fp8(1, None, 1, 1, 1, 1, 128, 64, 7, None)

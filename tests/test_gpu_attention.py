@@ -266,8 +266,38 @@ def test_custom_mask_operator_with_grouped_kv_heads(H, Hkv, D, dtype):
     o, sparsity = sa.block_sparse_sage2_attn_cuda(q, k, v, mask_id=mask.cuda(), pvthreshd=3.0, return_sparsity=True)
     assert o.shape == q.shape and abs(sparsity - res["sparsity"]) < 1e-6
     _check_out(o, res["out"])
-    with pytest.raises(RuntimeError, match="as many K heads"):
-        sa.spas_sage2_attn_meansim_topk_cuda(q, k, v)
+    with pytest.raises(ValueError, match="must be divisible by num_kv_heads"):
+        sa.spas_sage2_attn_meansim_topk_cuda(q, k[:, :1].expand(B, 4, N, D) if H == 6 else k[:, :1].expand(B, 3, N, D), v)
+
+
+@pytest.mark.parametrize("H,Hkv,D,dtype,causal", [(4, 2, 64, torch.float16, False), (6, 1, 128, torch.bfloat16, True),
+                                                   (8, 4, 128, torch.bfloat16, False)])
+def test_mask_prediction_with_grouped_kv_heads(H, Hkv, D, dtype, causal):
+    """Fewer K/V heads than query heads through the WHOLE operator (the reference's mask prediction needs equal head
+    counts, utils.py:388): K is pooled and quantised per K head, every query head of a group is scored against it with
+    its own top-k.  Block map, LUT and quantised tensors bit for bit against the oracle, output at tolerance."""
+    B, N = 1, 768
+    q = rand_T((B, H, N, D), dtype, 170)
+    k = rand_T((B, Hkv, N, D), dtype, 171, shift=0.3)
+    v = rand_T((B, Hkv, N, D), dtype, 172)
+    topk = torch.linspace(0.3, 0.8, H)
+    res = oapi.spas_sage2_attn_meansim_topk(to_np(q), to_np(k), to_np(v), tag_of(dtype), is_causal=causal, topk=topk.numpy())
+    km = _lib.km_mean(k)
+    bmap, q8, qs, k8, ks = utils.get_block_map_meansim_fuse_quant(q, k, km, is_causal=causal, simthreshd1=-0.1,
+                                                                  cdfthreshd=None, topk=topk.cuda())
+    assert k8.shape[1] == Hkv and np.array_equal(k8.cpu().numpy(), res["k8"]) and np.array_equal(q8.cpu().numpy(), res["q8"])
+    assert np.array_equal(bmap.cpu().numpy(), res["map"])
+    o, sp = sa.spas_sage2_attn_meansim_topk_cuda(q, k, v, is_causal=causal, topk=topk.cuda(), return_sparsity=True)
+    assert abs(sp - res["sparsity"]) < 1e-6
+    _check_out(o, res["out"])
+    # CDF selection and the INT8-QK / FP16-PV operator on the same shapes
+    res = oapi.spas_sage2_attn_meansim_topk(to_np(q), to_np(k), to_np(v), tag_of(dtype), simthreshd1=0.3, cdfthreshd=0.9,
+                                            topk=None)
+    o = sa.spas_sage2_attn_meansim_cuda(q, k, v, simthreshd1=0.3, cdfthreshd=0.9)
+    _check_out(o, res["out"])
+    res = oapi.spas_sage_attn_meansim_topk(to_np(q), to_np(k), to_np(v), tag_of(dtype), topk=0.5, is_causal=causal)
+    o = sa.spas_sage_attn_meansim_topk_cuda(q, k, v, topk=0.5, is_causal=causal)
+    _check_out(o, res["out"])
 
 
 @pytest.mark.parametrize("fp16v", [False, True])

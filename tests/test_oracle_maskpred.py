@@ -243,3 +243,23 @@ def test_map_to_lut_bruteforce_and_closed_form():
     # any non-zero value counts as set (float / negative entries)
     lut2, valid2 = mp.map_to_lut(np.where(m, -2.5, 0.0))
     assert np.array_equal(lut2, lut) and np.array_equal(valid2, valid)
+
+
+def test_grouped_kv_heads_equal_repeated_kv_heads():
+    """Mask prediction with fewer K heads than Q heads (an extension over utils.py:388): identical to multi-head
+    prediction on K repeated per group, for top-k and CDF selection with per-head hyper-parameters."""
+    from oracle import api
+    tag, d, n, H, Hkv = R.BF16, 64, 640, 4, 2
+    rng = np.random.default_rng(33)
+    mk = lambda h, s=1.0: R.round_to(rng.standard_normal((1, h, n, d)) * s, tag)
+    q, k, v = mk(H), mk(Hkv) + 0.3, mk(Hkv)
+    krep, vrep = np.repeat(k, H // Hkv, axis=1), np.repeat(v, H // Hkv, axis=1)
+    for kw in (dict(topk=np.array([0.5, 0.3, 0.7, 0.2], np.float32)),
+               dict(topk=None, cdfthreshd=np.array([0.9, 0.5, 0.97, 0.7], np.float32), simthreshd1=0.05, is_causal=True)):
+        g = api.spas_sage2_attn_meansim_topk(q, k, v, tag, **kw)
+        m = api.spas_sage2_attn_meansim_topk(q, krep, vrep, tag, **kw)
+        assert g["k8"].shape[1] == Hkv and g["map"].shape[1] == H
+        assert np.array_equal(g["map"], m["map"]) and np.array_equal(g["lut"], m["lut"])
+        assert np.array_equal(g["out"], m["out"])
+        if kw.get("topk") is not None:
+            assert not np.array_equal(g["map"][:, 0], g["map"][:, 1])      # heads of one group still select differently
