@@ -267,7 +267,8 @@ def test_custom_mask_operator_with_grouped_kv_heads(H, Hkv, D, dtype):
     assert o.shape == q.shape and abs(sparsity - res["sparsity"]) < 1e-6
     _check_out(o, res["out"])
     with pytest.raises(ValueError, match="must be divisible by num_kv_heads"):
-        sa.spas_sage2_attn_meansim_topk_cuda(q, k[:, :1].expand(B, 4, N, D) if H == 6 else k[:, :1].expand(B, 3, N, D), v)
+        bad = 4 if H == 6 else 3                        # a K/V head count that does not divide H
+        sa.spas_sage2_attn_meansim_topk_cuda(q, k[:, :1].expand(B, bad, N, D), v[:, :1].expand(B, bad, N, D))
 
 
 @pytest.mark.parametrize("H,Hkv,D,dtype,causal", [(4, 2, 64, torch.float16, False), (6, 1, 128, torch.bfloat16, True),
