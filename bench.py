@@ -292,6 +292,26 @@ def main():
                              "mfma_frac": dense_flop / dn / PEAK_MFMA_F16,
                              "speedup_step": dn / step_s, "speedup_attn_kernel": dn / attn_s,
                              "speedup_step_median": dense_stats["median"] / step_stats["median"]}
+        # an independent dense FP16 kernel for scale: PyTorch's own flash-attention backend on the same tensors (not
+        # part of this library; skipped when the backend refuses the shape or is missing)
+        try:
+            from torch.nn.attention import sdpa_kernel, SDPBackend
+            with sdpa_kernel([SDPBackend.FLASH_ATTENTION]):
+                sd = lambda: torch.nn.functional.scaled_dot_product_attention(qh, kh, vh, is_causal=cfg.is_causal)
+                for _ in range(2):
+                    sd()
+                torch.cuda.synchronize()
+                t0 = time.perf_counter()
+                for _ in range(max(3, args.steps // 2)):
+                    sd()
+                torch.cuda.synchronize()
+                ts = (time.perf_counter() - t0) / max(3, args.steps // 2)
+            out["dense_fp16"]["torch_sdpa_flash"] = {"ms": ts * 1e3, "tops": dense_flop / ts / 1e12,
+                                                     "speedup_step": ts / step_s,
+                                                     "note": "torch.nn.functional.scaled_dot_product_attention, "
+                                                             "FLASH_ATTENTION backend, fp16, same shape"}
+        except Exception as e:      # noqa: BLE001 - a missing backend must not break the bench line
+            out["dense_fp16"]["torch_sdpa_flash"] = {"ms": None, "note": f"not available: {type(e).__name__}"}
         del qh, kh, vh, vt, oh
 
     if not args.no_cpu_baseline:
