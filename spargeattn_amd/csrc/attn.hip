@@ -70,6 +70,14 @@ __device__ __forceinline__ void lds_read_2x128(v4i &a, v4i &b, uint32_t addr) {
                : "v"(addr), "n"(OFF0), "n"(OFF1)
                : "memory");
 }
+// two reads at the same immediate offset from two addresses (the two key chunks of a V^T row)
+template <int OFF>
+__device__ __forceinline__ void lds_read_pair(v4i &a, v4i &b, uint32_t addr_a, uint32_t addr_b) {
+  asm volatile("ds_read_b128 %0, %2 offset:%4\n\tds_read_b128 %1, %3 offset:%4"
+               : "=&v"(a), "=&v"(b)
+               : "v"(addr_a), "v"(addr_b), "n"(OFF)
+               : "memory");
+}
 // wait for all outstanding LDS reads; the operands tie the wait to the registers it makes valid
 __device__ __forceinline__ void lds_wait4(v4i &a, v4i &b, v4i &c, v4i &d) {
   asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(a), "+v"(b), "+v"(c), "+v"(d));
@@ -282,20 +290,36 @@ __global__ __launch_bounds__(256, PV16 ? 2 : 3) void block_sparse_attn_kernel(co
   // One K block.  TAIL = false: every block but the last two - PV-threshold test, no masks (sm89.cuh:283-391).
   // TAIL = true: the last two blocks - token-causal and out-of-bound masks, no skip (sm89.cuh:467-648).  The two are
   // separate loops so that the common one carries none of the tail's predicates.
-  auto step = [&](auto tail_tag, const int it) __attribute__((always_inline)) {
+  // SLOT = 0, 1, 2: the ring slot of the block is a compile-time constant (the common loop is unrolled three times), so
+  // every LDS address of the iteration is a loop-invariant register plus an immediate offset; SLOT = -1: the slot is the
+  // run-time value `bufoff` (the up to two left-over blocks of the common loop and the two tail blocks).
+  uint32_t kaddr_c[KS];
+#pragma unroll
+  for (int ks = 0; ks < KS; ks++) kaddr_c[ks] = lds_k0 + k_rd_base + ((uint32_t)(32 * ks) ^ k_rd_x);
+  const uint32_t va_lo_c = lds_v0 + v_rd_lo, va_hi_c = lds_v0 + (v_rd_lo ^ 16u);
+  const float cq = c * qs;                          // exponent multiplier = cq * k_scale of the block
+  const float cq26 = cq * SPG_ACC_SCALE;
+  // a 2^26 / (2 pi) >= 2^14  <=>  k_scale >= this bound; both are positive floats, so their bit patterns compare as integers
+  const int kscale_precise_bits = __builtin_bit_cast(int, 16384.0f / (acc_c * cq26));
+  auto step = [&](auto tail_tag, auto slot_tag, const int it) __attribute__((always_inline)) {
     constexpr bool TAIL = decltype(tail_tag)::value;
+    constexpr int SLOT = decltype(slot_tag)::value;
+    constexpr bool CS = SLOT >= 0 && !PV16;         // compile-time ring slot
     // ---- S^T = K . Q^T ---------------------------------------------------------------------------------
     v16i S0, S1;
     {
       // two groups of k-steps: the reads of the second group are in flight while the first group's MFMAs run
       constexpr int HK = KS / 2;
-      const uint32_t kaddr = lds_k0 + bufoff + k_rd_base;
       v4i a0[KS], a1[KS];
+      auto read_k = [&](int ks) __attribute__((always_inline)) {
+        if constexpr (CS) lds_read_2x128<(SLOT < 0 ? 0 : SLOT) * TILE, (SLOT < 0 ? 0 : SLOT) * TILE + 16 * D>(a0[ks], a1[ks], kaddr_c[ks]);
+        else lds_read_2x128<0, 16 * D>(a0[ks], a1[ks], kaddr_c[ks] + bufoff);
+      };
 #pragma unroll
-      for (int ks = 0; ks < HK; ks++) lds_read_2x128<0, 16 * D>(a0[ks], a1[ks], kaddr + ((uint32_t)(32 * ks) ^ k_rd_x));
+      for (int ks = 0; ks < HK; ks++) read_k(ks);
       if constexpr (HK == 2) lds_wait4(a0[0], a1[0], a0[1], a1[1]); else lds_wait2(a0[0], a1[0]);
 #pragma unroll
-      for (int ks = HK; ks < KS; ks++) lds_read_2x128<0, 16 * D>(a0[ks], a1[ks], kaddr + ((uint32_t)(32 * ks) ^ k_rd_x));
+      for (int ks = HK; ks < KS; ks++) read_k(ks);
       // the first product of each chain, with the inline constant as its C operand (the compiler would otherwise keep
       // the constant in sixteen registers); the products that follow accumulate onto these and are ordinary builtins,
       // which the other chain's product always separates from their predecessor
@@ -326,16 +350,16 @@ __global__ __launch_bounds__(256, PV16 ? 2 : 3) void block_sparse_attn_kernel(co
       d4 = it + 4 < nv ? lutc[it + 4] : 0;
     }
     __builtin_amdgcn_sched_barrier(0);
-    const float dq = qs * ksc;
+    const float dq = qs * ksc;                     // used by the tail blocks only
     // S0/S1 are never rewritten (no copies at the join of the two paths): slot e < 16 is S0[e], slot e >= 16 is S1[e - 16]
-    const float a = c * dq;
-    const float a26 = a * SPG_ACC_SCALE;           // multiplier of the accumulator read as a float (exact scaling)
+    const float a = cq * ksc;
+    const float a26 = cq26 * ksc;                  // multiplier of the accumulator read as a float
     // The constant 1/(2 pi) leaves the exponent through ONE additive term, -(1/(2 pi) a 2^26 + m) (+ 8.807), whose rounding
     // error is half an ulp of 1.07e7 a.  Below 2^14 that is at most 2^-11 in the exponent (3e-4 relative in P, and the
     // row maximum's P stays below 448.2).  At or above it (large |q| |k| or a large softmax scale; uniform for the
     // workgroup) the scores are first taken relative to the lane's own maximum - an exact subtraction inside one binade -
     // so that no large constant is left to round: one more instruction per score, on such blocks only.
-    const bool precise = a26 * acc_c >= 16384.0f;
+    const bool precise = __builtin_bit_cast(int, ksc) >= kscale_precise_bits;
     float fm, mloc = acc_c;
     int lim = 0x7fffffff;
     if constexpr (!TAIL) {
@@ -383,8 +407,12 @@ __global__ __launch_bounds__(256, PV16 ? 2 : 3) void block_sparse_attn_kernel(co
         compute = (sVote[it & 1][0] | sVote[it & 1][1] | sVote[it & 1][2] | sVote[it & 1][3]) != 0;
     }
     if (!TAIL || it + 2 < nv) {
-      const uint32_t b2 = bufoff == 0 ? 2 * TILE : bufoff - TILE;   // slot (it+2) % 3
-      SPG_LOAD_TILES(blk2, b2);
+      if constexpr (CS) {
+        SPG_LOAD_TILES(blk2, ((SLOT + 2) % 3) * TILE);
+      } else {
+        const uint32_t b2 = bufoff == 0 ? 2 * TILE : bufoff - TILE;   // slot (it+2) % 3
+        SPG_LOAD_TILES(blk2, b2);
+      }
     }
     dsum *= osc;
     if (__any(osc != 1.0f)) {
@@ -492,19 +520,19 @@ __global__ __launch_bounds__(256, PV16 ? 2 : 3) void block_sparse_attn_kernel(co
       for (int u = 0; u < 8; u++) pb[u] = pack4_e4m3(x[4 * u], x[4 * u + 1], x[4 * u + 2], x[4 * u + 3]);
       {
         constexpr int HD = NDT / 2;
-        const uint32_t va_lo = lds_v0 + bufoff + v_rd_lo, va_hi = lds_v0 + bufoff + (v_rd_lo ^ 16u);
+        constexpr int SB = CS ? SLOT * TILE : 0;     // ring slot as an immediate, or in the address registers
+        const uint32_t va_lo = CS ? va_lo_c : va_lo_c + bufoff, va_hi = CS ? va_hi_c : va_hi_c + bufoff;
         v4i lo[NDT], hi[NDT];
-        // group 0
-        asm volatile("ds_read_b128 %0, %2\n\tds_read_b128 %1, %3" : "=&v"(lo[0]), "=&v"(hi[0]) : "v"(va_lo), "v"(va_hi) : "memory");
-        if constexpr (HD == 2)
-          asm volatile("ds_read_b128 %0, %2 offset:2048\n\tds_read_b128 %1, %3 offset:2048" : "=&v"(lo[1]), "=&v"(hi[1]) : "v"(va_lo), "v"(va_hi) : "memory");
+        // group 0 (output tile dt reads channel rows 32 dt .. 32 dt + 31: 2048 bytes further on)
+        lds_read_pair<SB>(lo[0], hi[0], va_lo, va_hi);
+        if constexpr (HD == 2) lds_read_pair<SB + 2048>(lo[1], hi[1], va_lo, va_hi);
         if constexpr (HD == 2) lds_wait4(lo[0], hi[0], lo[1], hi[1]); else lds_wait2(lo[0], hi[0]);
         // group 1 in flight while group 0 multiplies
         if constexpr (HD == 2) {
-          asm volatile("ds_read_b128 %0, %2 offset:4096\n\tds_read_b128 %1, %3 offset:4096" : "=&v"(lo[2]), "=&v"(hi[2]) : "v"(va_lo), "v"(va_hi) : "memory");
-          asm volatile("ds_read_b128 %0, %2 offset:6144\n\tds_read_b128 %1, %3 offset:6144" : "=&v"(lo[3]), "=&v"(hi[3]) : "v"(va_lo), "v"(va_hi) : "memory");
+          lds_read_pair<SB + 4096>(lo[2], hi[2], va_lo, va_hi);
+          lds_read_pair<SB + 6144>(lo[3], hi[3], va_lo, va_hi);
         } else {
-          asm volatile("ds_read_b128 %0, %2 offset:2048\n\tds_read_b128 %1, %3 offset:2048" : "=&v"(lo[1]), "=&v"(hi[1]) : "v"(va_lo), "v"(va_hi) : "memory");
+          lds_read_pair<SB + 2048>(lo[1], hi[1], va_lo, va_hi);
         }
 #pragma unroll
         for (int dt = 0; dt < HD; dt++) {
@@ -523,14 +551,22 @@ __global__ __launch_bounds__(256, PV16 ? 2 : 3) void block_sparse_attn_kernel(co
     // advance the block pipeline and the ring
     blk = blk1; blk1 = blk2; blk2 = blk2 + d3; d3 = d4;
     ksc = ksc1; ksc1 = ksc2;
-    bufoff = bufoff == 2 * TILE ? 0 : bufoff + TILE;
+    if constexpr (!CS) bufoff = bufoff == 2 * TILE ? 0 : bufoff + TILE;
   };
   {
     int it = 0;
+    // the common loop, three blocks per trip (ring slots 0, 1, 2); `bufoff` stays 0 throughout where the slots are
+    // compile-time constants, and three run-time steps bring it back to 0 where they are not
 #pragma unroll 1
-    for (; it < nv - 2; it++) step(std::false_type{}, it);
+    for (; it + 3 <= nv - 2; it += 3) {
+      step(std::false_type{}, std::integral_constant<int, 0>{}, it);
+      step(std::false_type{}, std::integral_constant<int, 1>{}, it + 1);
+      step(std::false_type{}, std::integral_constant<int, 2>{}, it + 2);
+    }
 #pragma unroll 1
-    for (; it < nv; it++) step(std::true_type{}, it);
+    for (; it < nv - 2; it++) step(std::false_type{}, std::integral_constant<int, -1>{}, it);
+#pragma unroll 1
+    for (; it < nv; it++) step(std::true_type{}, std::integral_constant<int, -1>{}, it);
   }
 #undef SPG_LOAD_TILES
 #undef SPG_LANE_OFFSETS
