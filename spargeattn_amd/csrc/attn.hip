@@ -78,6 +78,20 @@ __device__ __forceinline__ void lds_read_pair(v4i &a, v4i &b, uint32_t addr_a, u
                : "v"(addr_a), "v"(addr_b), "n"(OFF)
                : "memory");
 }
+// v_max_f32 as one instruction: fmaxf() on a value the compiler cannot prove to be a quiet number (a loop-carried
+// maximum, the output of a lane exchange) costs a canonicalising self-maximum per operand first.  The operands here are
+// products and maxima of finite numbers.
+__device__ __forceinline__ float max_raw(float a, float b) {
+  float r;
+  asm("v_max_f32 %0, %1, %2" : "=v"(r) : "v"(a), "v"(b));
+  return r;
+}
+__device__ __forceinline__ float half_swap_max_raw(float v) {
+  float lo, hi, r;
+  half_swap(v, lo, hi);
+  asm("s_nop 0\n\tv_max_f32 %0, %1, %2" : "=v"(r) : "v"(lo), "v"(hi));   // one idle state behind the lane exchange
+  return r;
+}
 // wait for all outstanding LDS reads; the operands tie the wait to the registers it makes valid
 __device__ __forceinline__ void lds_wait4(v4i &a, v4i &b, v4i &c, v4i &d) {
   asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(a), "+v"(b), "+v"(c), "+v"(d));
@@ -297,8 +311,7 @@ __global__ __launch_bounds__(256, PV16 ? 2 : 3) void block_sparse_attn_kernel(co
 #pragma unroll
   for (int ks = 0; ks < KS; ks++) kaddr_c[ks] = lds_k0 + k_rd_base + ((uint32_t)(32 * ks) ^ k_rd_x);
   const uint32_t va_lo_c = lds_v0 + v_rd_lo, va_hi_c = lds_v0 + (v_rd_lo ^ 16u);
-  const float cq = c * qs;                          // exponent multiplier = cq * k_scale of the block
-  const float cq26 = cq * SPG_ACC_SCALE;
+  const float cq26 = c * qs * SPG_ACC_SCALE;        // exponent multiplier a of a block = cq26 * k_scale * 2^-26
   // a 2^26 / (2 pi) >= 2^14  <=>  k_scale >= this bound; both are positive floats, so their bit patterns compare as integers
   const int kscale_precise_bits = __builtin_bit_cast(int, 16384.0f / (acc_c * cq26));
   auto step = [&](auto tail_tag, auto slot_tag, const int it) __attribute__((always_inline)) {
@@ -352,8 +365,7 @@ __global__ __launch_bounds__(256, PV16 ? 2 : 3) void block_sparse_attn_kernel(co
     __builtin_amdgcn_sched_barrier(0);
     const float dq = qs * ksc;                     // used by the tail blocks only
     // S0/S1 are never rewritten (no copies at the join of the two paths): slot e < 16 is S0[e], slot e >= 16 is S1[e - 16]
-    const float a = cq * ksc;
-    const float a26 = cq26 * ksc;                  // multiplier of the accumulator read as a float
+    const float a26 = cq26 * ksc;                  // multiplier of the accumulator read as a float: a * 2^26
     // The constant 1/(2 pi) leaves the exponent through ONE additive term, -(1/(2 pi) a 2^26 + m) (+ 8.807), whose rounding
     // error is half an ulp of 1.07e7 a.  Below 2^14 that is at most 2^-11 in the exponent (3e-4 relative in P, and the
     // row maximum's P stays below 448.2).  At or above it (large |q| |k| or a large softmax scale; uniform for the
@@ -368,8 +380,8 @@ __global__ __launch_bounds__(256, PV16 ? 2 : 3) void block_sparse_attn_kernel(co
       for (int e = 1; e < 16; e++) imax = max(imax, S0[e]);
 #pragma unroll
       for (int e = 0; e < 16; e++) imax = max(imax, S1[e]);
-      fm = (float)(imax - SPG_ACC_C_BITS) * a;
       mloc = __builtin_bit_cast(float, imax);   // 1/(2 pi) + 2^-26 * the largest of this lane's 32 dot products
+      fm = (mloc - acc_c) * a26;                // the subtraction is exact (same binade)
     } else {
       // slot e of this lane is key 64*blk + 32*hh + e; keys beyond `lim` are masked
       const int key0 = blk * 64 + 32 * hh;
@@ -385,9 +397,9 @@ __global__ __launch_bounds__(256, PV16 ? 2 : 3) void block_sparse_attn_kernel(co
       }
       fm = fm * c;
     }
-    fm = half_swap_max_f32(fm);
+    fm = half_swap_max_raw(fm);
     const float diff = fm - m;
-    const float m_new = fmaxf(m, fm);
+    const float m_new = max_raw(m, fm);
     const float osc = __builtin_amdgcn_exp2f(m - m_new);
     m = m_new;
     int vote = 1;
