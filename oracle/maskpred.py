@@ -246,6 +246,12 @@ def num_to_select_topk(topk, nk):
 def num_to_select_cdf(p, order, cdfthreshd, dtype):
     """cumsum of the sorted probabilities rounded to T, then searchsorted(right=True) (utils.py:398-403).
 
+    PARITY UNPINNED: cdf[i] is defined here as the EXACT running sum rounded once to T.  The reference calls
+    torch.cumsum on a bf16/fp16 CUDA tensor, whose scan may combine partial sums in the tensor dtype (a rounding per
+    combine step, in an order the library chooses); no fixture of the reference covers it.  On long bf16 rows such a
+    scan can stall below 1 and then counts MORE blocks for the same threshold, so a cdfthreshd tuned with the CUDA
+    reference may select a different number of blocks here.
+
     p (B,H,nq,nk); cdfthreshd (H,) float32.  Returns int64 (B,H,nq).
     """
     ps = np.take_along_axis(np.asarray(p, F64), order, axis=-1)

@@ -1,9 +1,10 @@
-"""Full-size GPU checks on the four large benchmark configurations (cfg2-cfg5 of spargeattn_amd/workloads.py) through size-independent properties.
+"""Full-size GPU checks on the four large benchmark configurations (cfg2-cfg5 of spargeattn_amd/workloads.py).
 
-The oracle is too slow at these sizes; instead each test checks invariants the algorithm fixes (row counts of the
-block map, LUT sortedness, quantisation round-trip bounds, code-range of the FP8 tensor, determinism) and compares
-sampled Q blocks of the attention output with a float32 torch computation on the de-quantised tensors under the
-token mask the LUT encodes.
+With every head the oracle is too slow at these sizes: those tests check invariants the algorithm fixes (row counts
+of the block map, LUT sortedness, quantisation round-trip bounds, code-range of the FP8 tensor, determinism) and
+compare sampled Q blocks of the attention output with a float32 torch computation on the de-quantised tensors under
+the token mask the LUT encodes.  ONE head at the full sequence length is within the oracle's reach (seconds): the last
+test compares every stage of cfg4 and cfg3 with it, bit for bit where the stage is exact.
 """
 import numpy as np
 import pytest
