@@ -214,12 +214,19 @@ __global__ __launch_bounds__(256, PV16 ? 2 : 3) void block_sparse_attn_kernel(co
   // u*1024 is the LDS offset: it rides in the instruction's immediate (applied to both addresses).
   // (the two per-lane offsets are recomputed from the thread id where they are used: cheaper than keeping them
   //  in registers across the loop, where the register file is the scarce resource)
+  // Split into a part that depends on the lane only (recomputed with three or four vector instructions where it is
+  // used) and a wavefront-uniform part that the compiler keeps in scalar registers: the K-row swizzle of chunk position
+  // pos = WL*64*wave + lane takes its bits from lane bits 4-5 (D = 128) or 4 (D = 64) and from bit 1 of the wave index.
+  static_assert(D == 64 || D == 128, "swizzle bit positions below");
+  const uint32_t kswz_wave16 = (uint32_t)((wave >> 1) & 1) << (D == 128 ? 6 : 5);
+  const uint32_t k_wave = (uint32_t)(WL * 1024 * wave), v_wave = (uint32_t)(WLV * 1024 * wave);
 #define SPG_LANE_OFFSETS()                                                                                    \
   uint32_t lane_ = threadIdx.x & 63u;                                                                         \
   asm volatile("" : "+v"(lane_));                                                                             \
   const uint32_t pos0 = (uint32_t)(WL * 64 * wave) + lane_;                                                   \
-  const uint32_t v_lane = ((uint32_t)(WLV * 64 * wave) + lane_) * 16u;                                        \
-  const uint32_t k_lane = (pos0 * 16u) ^ (k_swz<D>(pos0 / CPR) * 16u);   /* row * D + (slot ^ swz) * 16 */
+  const uint32_t v_lane = v_wave + lane_ * 16u;                                                               \
+  const uint32_t kswz_lane = D == 128 ? ((lane_ >> 4) & 3u) : ((lane_ >> 4) & 1u);                            \
+  const uint32_t k_lane = k_wave + (((lane_ ^ kswz_lane) << 4) ^ kswz_wave16);   /* row * D + (slot ^ swz) * 16 */
   const int last_partial_blk = (Nk % 64) ? p.nk - 1 : -1;   // the only block with rows beyond Nk
   typedef __attribute__((address_space(3))) void *lds_ptr_t;
   typedef const __attribute__((address_space(1))) void *glb_ptr_t;
