@@ -113,6 +113,40 @@ __global__ __launch_bounds__(256) void div_selftest_kernel(unsigned long long *c
   atomicAdd(&counts[1], bad);
 }
 
+// Packed 16-bit helpers.  A tile is kept in registers as the 16-bit patterns it was loaded with (two per register) and
+// widened where it is used: half the registers of a binary32 copy, which is what lets enough workgroups share a CU to
+// keep HBM busy.
+typedef unsigned short u16x2_t __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ uint32_t pk_max_u16(uint32_t a, uint32_t b) {
+  return __builtin_bit_cast(uint32_t, __builtin_elementwise_max(__builtin_bit_cast(u16x2_t, a), __builtin_bit_cast(u16x2_t, b)));
+}
+template <int DT> __device__ __forceinline__ void unpack2(uint32_t w, float &lo, float &hi) {
+  lo = elem_to_f32<DT>((uint16_t)(w & 0xffffu));
+  hi = elem_to_f32<DT>((uint16_t)(w >> 16));
+}
+// two binary32 values -> two 16-bit patterns, round to nearest even
+template <int DT> __device__ __forceinline__ uint32_t pack_round2(float a, float b);
+template <> __device__ __forceinline__ uint32_t pack_round2<0>(float a, float b) {
+  typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+  typedef float f2 __attribute__((ext_vector_type(2)));
+  const f2 v = {a, b};
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, h2));
+}
+template <> __device__ __forceinline__ uint32_t pack_round2<1>(float a, float b) {
+  typedef __bf16 bf2 __attribute__((ext_vector_type(2)));
+  typedef float f2 __attribute__((ext_vector_type(2)));
+  const f2 v = {a, b};
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf2));   // v_cvt_pk_bf16_f32
+}
+// Hides a register's value from the optimiser: placed between two passes over the packed tile, it keeps the compiler
+// from carrying the widened (binary32) copies of one pass over to the next, which would double the registers again.
+__device__ __forceinline__ void forget(uint32_t &v) { asm volatile("" : "+v"(v)); }
+__device__ __forceinline__ uint32_t wave_max_u32(uint32_t v) {
+#pragma unroll
+  for (int o = 32; o >= 1; o >>= 1) v = max(v, (uint32_t)__shfl_xor((int)v, o, SPG_WAVE));
+  return v;
+}
+
 template <int BS, int D, int DT, bool HAS_MEAN, bool WITH_POOL>
 __global__ __launch_bounds__(256) void pool_sim_quant_kernel(const uint16_t *__restrict__ x, const Strides xs,
                                                              const uint16_t *__restrict__ km,
@@ -122,67 +156,92 @@ __global__ __launch_bounds__(256) void pool_sim_quant_kernel(const uint16_t *__r
   constexpr int TPR = D / 8;
   constexpr int RPP = 256 / TPR;
   constexpr int NP = BS / RPP;
+  // magnitude patterns (sign bit cleared) order like the magnitudes, for both 16-bit formats
+  constexpr uint32_t ABS2 = 0x7fff7fffu;
+  constexpr uint32_t INF16 = DT == 1 ? 0x7f80u : 0x7c00u;
+  // "every element of the row is tiny": bfloat16 below 2^-63 (both top exponent bits clear), binary16 zero
+  constexpr uint32_t TINY2 = DT == 1 ? 0x60006000u : 0x7fff7fffu;
   const int blk = blockIdx.x, bh = blockIdx.y;
   const int tid = threadIdx.x, c = tid % TPR, r = tid / TPR;
   const int row_base = blk * BS;
   const int rows_valid = min(BS, N - row_base);
+  const bool partial = rows_valid < BS;          // workgroup-uniform: only the last block of a head
   const uint16_t *xb = x + (size_t)(bh / H) * xs.sb + (size_t)(bh % H) * xs.sh + (size_t)row_base * xs.sn + c * 8;
 
   float kmf[8];
   if constexpr (HAS_MEAN) {
     const uint4 v = *(const uint4 *)(km + (size_t)bh * D + c * 8);
-    const uint32_t w[4] = {v.x, v.y, v.z, v.w};
-#pragma unroll
-    for (int e = 0; e < 4; e++) {
-      kmf[2 * e] = elem_to_f32<DT>((uint16_t)(w[e] & 0xffffu));
-      kmf[2 * e + 1] = elem_to_f32<DT>((uint16_t)(w[e] >> 16));
-    }
+    unpack2<DT>(v.x, kmf[0], kmf[1]);
+    unpack2<DT>(v.y, kmf[2], kmf[3]);
+    unpack2<DT>(v.z, kmf[4], kmf[5]);
+    unpack2<DT>(v.w, kmf[6], kmf[7]);
   }
 
   // all loads of the thread are issued before the first use (rows beyond the block's end re-read its last row and
   // are zeroed afterwards: no load sits behind a branch)
-  uint4 raw[NP];
+  uint32_t w[NP][4];
+  {
+    uint4 raw[NP];
 #pragma unroll
-  for (int p = 0; p < NP; p++) raw[p] = *(const uint4 *)(xb + (size_t)min(r + p * RPP, rows_valid - 1) * xs.sn);
-  float xf[NP][8];
-  float amax = 0.f;
+    for (int p = 0; p < NP; p++) raw[p] = *(const uint4 *)(xb + (size_t)min(r + p * RPP, rows_valid - 1) * xs.sn);
 #pragma unroll
-  for (int p = 0; p < NP; p++) {
-    const int row = r + p * RPP;
-    const bool ok = row < rows_valid;
-    const uint4 v = ok ? raw[p] : make_uint4(0, 0, 0, 0);
-    const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+    for (int p = 0; p < NP; p++) { w[p][0] = raw[p].x; w[p][1] = raw[p].y; w[p][2] = raw[p].z; w[p][3] = raw[p].w; }
+  }
+  if constexpr (HAS_MEAN) {
+    // (k - km) rounded once to the input dtype (utils.py:184-188).  The binary32 difference of two 16-bit floats is
+    // either exact or nowhere near a rounding tie of the 16-bit format, so rounding it to nearest even equals rounding
+    // the exact difference.  The tile is kept as the rounded 16-bit patterns.
 #pragma unroll
-    for (int e = 0; e < 8; e += 2) {
-      float f0 = elem_to_f32<DT>((uint16_t)(w[e >> 1] & 0xffffu));
-      float f1 = elem_to_f32<DT>((uint16_t)(w[e >> 1] >> 16));
-      if constexpr (HAS_MEAN) {
-        // (k - km) rounded once to the input dtype (utils.py:184-188).  The binary32 difference of two 16-bit
-        // floats is either exact or nowhere near a rounding tie of the 16-bit format, so rounding it to nearest
-        // even equals rounding the exact difference.  Masked rows stay zero.
-        if (ok) {
-          f0 -= kmf[e];
-          f1 -= kmf[e + 1];
-          round2_through_elem<DT>(f0, f1);
-        }
+    for (int p = 0; p < NP; p++)
+#pragma unroll
+      for (int j = 0; j < 4; j++) {
+        float f0, f1;
+        unpack2<DT>(w[p][j], f0, f1);
+        w[p][j] = pack_round2<DT>(f0 - kmf[2 * j], f1 - kmf[2 * j + 1]);
       }
-      xf[p][e] = f0;
-      xf[p][e + 1] = f1;
-      amax = fmaxf(amax, fmaxf(fabsf(f0), fabsf(f1)));
-    }
+  }
+  if (partial) {                                  // masked rows are zero (utils.py:188)
+#pragma unroll
+    for (int p = 0; p < NP; p++)
+      if (r + p * RPP >= rows_valid) { w[p][0] = 0; w[p][1] = 0; w[p][2] = 0; w[p][3] = 0; }
   }
 
-  __shared__ float s_wmax[4];
+  // largest magnitude of the thread's elements (as a 16-bit pattern) and, per row, whether all of them are tiny
+  uint32_t m2 = 0, tiny_rows = 0;
+#pragma unroll
+  for (int p = 0; p < NP; p++) {
+    const uint32_t rm = pk_max_u16(pk_max_u16(w[p][0] & ABS2, w[p][1] & ABS2), pk_max_u16(w[p][2] & ABS2, w[p][3] & ABS2));
+    m2 = pk_max_u16(m2, rm);
+    if constexpr (WITH_POOL) tiny_rows |= ((rm & TINY2) == 0 ? 1u : 0u) << p;
+  }
+  const uint32_t m_thread = max(m2 & 0xffffu, m2 >> 16);
+  __shared__ uint32_t s_wmax[4];
   __shared__ long long s_wg[4];
-  amax = wave_max_f32(amax);
-  if ((tid & 63) == 0) s_wmax[tid >> 6] = amax;
+  {
+    const uint32_t mw = wave_max_u32(m_thread);
+    if ((tid & 63) == 0) s_wmax[tid >> 6] = mw;
+  }
 
   if constexpr (WITH_POOL) {
     __shared__ double s_col[RPP][D];
     __shared__ double s_xh[RPP][D];
-    double colsum[8], colxh[8];
+    double colsum[8];
 #pragma unroll
-    for (int e = 0; e < 8; e++) { colsum[e] = 0.0; colxh[e] = 0.0; }
+    for (int e = 0; e < 8; e++) colsum[e] = 0.0;
+    // column sums for the pooled mean: binary64, exact
+#pragma unroll
+    for (int p = 0; p < NP; p++)
+#pragma unroll
+      for (int j = 0; j < 4; j++) {
+        float f0, f1;
+        forget(w[p][j]);
+        unpack2<DT>(w[p][j], f0, f1);
+        colsum[2 * j] += (double)f0;
+        colsum[2 * j + 1] += (double)f1;
+      }
+#pragma unroll
+    for (int e = 0; e < 8; e++) s_col[r][c * 8 + e] = colsum[e];
+
     // row norms: the TPR lanes of a row group all need sqrt(sum of squares) and its reciprocal for each of their NP
     // rows.  Both are computed ONCE per NP rows - lane c of the group takes row c % NP - and handed round with lane
     // reads, instead of NP times in every lane.
@@ -191,31 +250,18 @@ __global__ __launch_bounds__(256) void pool_sim_quant_kernel(const uint16_t *__r
     // the statistic is ||sum of x_hat||^2 / rows^2 >= 0 > threshold whenever every x_hat is finite.  x_hat = x / norm is
     // non-finite exactly for rows with norm == 0 (all-zero rows such as the padding of a partial block, or rows too
     // small for their squares) and for non-finite x; |x| <= norm (1 + 2^-23) keeps every other quotient within fp16.
+    // Only two facts about the rows are needed then: is any element non-finite, and does any row have a zero norm.  A
+    // row whose largest |x| is at least 2^-63 has a sum of squares of at least 2^-126, a positive binary32 number; rows
+    // in which every element is smaller (all-zero rows, the padding of a partial block, bfloat16 values near the bottom
+    // of the range) are decided by the exact sums below.
     const bool sim_trivial = simthr[bh % H] < 0.f;     // workgroup-uniform
     int bad_rows = 0;
     float ssf_mine = 0.f;
-    // Column sums for the pooled mean (binary64), and - with a negative threshold - a scan of the bit patterns:
-    // only two facts about the rows are needed then, is any element non-finite and does any row have a zero norm.
-    // A row whose largest |x| is at least 2^-74 has a sum of squares of at least 2^-148, which rounds to a positive
-    // binary32 number; rows in which every element is smaller than that (all-zero rows, the padding of a partial block,
-    // bf16 values near the bottom of the range) are decided by the exact sums below.
-    uint32_t abs_max = 0, tiny_rows = 0;
-#pragma unroll
-    for (int p = 0; p < NP; p++) {
-      uint32_t m = 0;
-#pragma unroll
-      for (int e = 0; e < 8; e++) {
-        colsum[e] += (double)xf[p][e];
-        m = max(m, __builtin_bit_cast(uint32_t, xf[p][e]) & 0x7fffffffu);
-      }
-      abs_max = max(abs_max, m);
-      tiny_rows |= (m < 0x1A800000u ? 1u : 0u) << p;        // 0x1A800000 = 2^-74
-    }
-    bool need_norms = true;                                  // wavefront-uniform
+    bool need_norms = true;                            // wavefront-uniform
     if (sim_trivial) {
-      bad_rows |= abs_max >= 0x7f800000u ? 1 : 0;           // inf or NaN anywhere (overflowing squares of finite values are harmless: x / inf = 0)
-      tiny_rows = group_and_u32<TPR>(tiny_rows);            // rows tiny in every lane of their group
-      need_norms = __any(tiny_rows != 0);                   // rare
+      bad_rows |= m_thread >= INF16 ? 1 : 0;          // inf or NaN anywhere (overflowing squares of finite values are harmless: x / inf = 0)
+      tiny_rows = group_and_u32<TPR>(tiny_rows);      // rows tiny in every lane of their group
+      need_norms = __any(tiny_rows != 0);             // rare
     }
     if (need_norms) {
       // sum of squares of every row (exact in binary64), rounded to binary32 like the reference's (utils.py:194)
@@ -223,9 +269,13 @@ __global__ __launch_bounds__(256) void pool_sim_quant_kernel(const uint16_t *__r
       for (int p = 0; p < NP; p++) {
         double ss = 0.0;
 #pragma unroll
-        for (int e = 0; e < 8; e++) {
-          const double xd = (double)xf[p][e];
-          ss = __builtin_fma(xd, xd, ss);             // squares and their sum are exact in binary64
+        for (int j = 0; j < 4; j++) {
+          float f0, f1;
+          forget(w[p][j]);
+          unpack2<DT>(w[p][j], f0, f1);
+          const double d0 = (double)f0, d1 = (double)f1;
+          ss = __builtin_fma(d0, d0, ss);             // squares and their sum are exact in binary64
+          ss = __builtin_fma(d1, d1, ss);
         }
         ss = group_sum_f64<TPR>(ss);                 // the TPR lanes of this row
         const float ssf = (float)ss;
@@ -234,31 +284,29 @@ __global__ __launch_bounds__(256) void pool_sim_quant_kernel(const uint16_t *__r
       }
     }
     if (!sim_trivial) {
-    const float norm_mine = sqrtf(ssf_mine);
-    const float rn_mine = rcp_safe(norm_mine) ? exact_rcp(norm_mine) : 0.f;
-    const int group_lane0 = (tid & 63) & ~(TPR - 1);
+      double colxh[8];
 #pragma unroll
-    for (int p = 0; p < NP; p++) {
-      const float norm = __shfl(norm_mine, group_lane0 + p, SPG_WAVE);
-      const float rn = __shfl(rn_mine, group_lane0 + p, SPG_WAVE);
-      if (rcp_safe(norm)) {
+      for (int e = 0; e < 8; e++) colxh[e] = 0.0;
+      const float norm_mine = sqrtf(ssf_mine);
+      const float rn_mine = rcp_safe(norm_mine) ? exact_rcp(norm_mine) : 0.f;
+      const int group_lane0 = (tid & 63) & ~(TPR - 1);
 #pragma unroll
-        for (int e = 0; e < 8; e++) {
-          const _Float16 h = (_Float16)div_by(xf[p][e], norm, rn);
-          colxh[e] += (double)(float)h;             // fp16 values: integer multiples of 2^-24, sums are exact
-        }
-      } else {
+      for (int p = 0; p < NP; p++) {
+        const float norm = __shfl(norm_mine, group_lane0 + p, SPG_WAVE);
+        const float rn = __shfl(rn_mine, group_lane0 + p, SPG_WAVE);
+        const bool fast = rcp_safe(norm);
 #pragma unroll
-        for (int e = 0; e < 8; e++) {
-          const _Float16 h = (_Float16)(xf[p][e] / norm);   // 0/0 -> NaN for all-zero (masked) rows
-          colxh[e] += (double)(float)h;
+        for (int j = 0; j < 4; j++) {
+          float f0, f1;
+          forget(w[p][j]);
+          unpack2<DT>(w[p][j], f0, f1);
+          // 0/0 -> NaN for all-zero (masked) rows on the slow branch
+          const _Float16 h0 = (_Float16)(fast ? div_by(f0, norm, rn) : f0 / norm);
+          const _Float16 h1 = (_Float16)(fast ? div_by(f1, norm, rn) : f1 / norm);
+          colxh[2 * j] += (double)(float)h0;          // fp16 values: integer multiples of 2^-24, sums are exact
+          colxh[2 * j + 1] += (double)(float)h1;
         }
       }
-    }
-    }   // !sim_trivial
-#pragma unroll
-    for (int e = 0; e < 8; e++) s_col[r][c * 8 + e] = colsum[e];
-    if (!sim_trivial) {
 #pragma unroll
       for (int e = 0; e < 8; e++) s_xh[r][c * 8 + e] = colxh[e];
     }
@@ -293,21 +341,29 @@ __global__ __launch_bounds__(256) void pool_sim_quant_kernel(const uint16_t *__r
     __syncthreads();
   }
 
-  amax = fmaxf(fmaxf(s_wmax[0], s_wmax[1]), fmaxf(s_wmax[2], s_wmax[3]));
+  const uint32_t m_blk = max(max(s_wmax[0], s_wmax[1]), max(s_wmax[2], s_wmax[3]));
+  const float amax = elem_to_f32<DT>((uint16_t)m_blk);
   const float s = amax / 127.0f + 1e-7f;
   int8_t *qb = xq + ((size_t)bh * N + row_base) * D + c * 8;
   auto quantise = [&](auto divide) {
 #pragma unroll
     for (int p = 0; p < NP; p++) {
       const int row = r + p * RPP;
-      if (row < rows_valid) {
+      if (!partial || row < rows_valid) {
         uint32_t pk[2] = {0, 0};
 #pragma unroll
-        for (int e = 0; e < 8; e++) {
-          float y = divide(xf[p][e]);
-          y = y + __builtin_copysignf(0.5f, y);   // +0.5 for y >= 0 (a -0 quotient truncates to 0 either way)
-          const int q = (int)y;   // truncation toward zero
-          pk[e >> 2] |= ((uint32_t)q & 0xffu) << (8 * (e & 3));
+        for (int j = 0; j < 4; j++) {
+          float f[2];
+          forget(w[p][j]);
+          unpack2<DT>(w[p][j], f[0], f[1]);
+#pragma unroll
+          for (int h = 0; h < 2; h++) {
+            float y = divide(f[h]);
+            y = y + __builtin_copysignf(0.5f, y);   // +0.5 for y >= 0 (a -0 quotient truncates to 0 either way)
+            const int q = (int)y;   // truncation toward zero
+            const int e = 2 * j + h;
+            pk[e >> 2] |= ((uint32_t)q & 0xffu) << (8 * (e & 3));
+          }
         }
         *(uint2 *)(qb + (size_t)row * D) = make_uint2(pk[0], pk[1]);
       }
