@@ -18,6 +18,7 @@
 #include "launch.h"
 
 #include <atomic>
+#include <type_traits>
 
 namespace spg {
 
@@ -147,25 +148,35 @@ __device__ __forceinline__ uint32_t wave_max_u32(uint32_t v) {
   return v;
 }
 
+// One workgroup handles 128 consecutive rows of one (batch, head): one 128-row block or two 64-row blocks (SUB), so
+// that the per-block tail (column reduction, pooled mean, flag, scale) is spread over all four wavefronts in both cases.
 template <int BS, int D, int DT, bool HAS_MEAN, bool WITH_POOL>
 __global__ __launch_bounds__(256) void pool_sim_quant_kernel(const uint16_t *__restrict__ x, const Strides xs,
                                                              const uint16_t *__restrict__ km,
                                                              uint16_t *__restrict__ pool, uint8_t *__restrict__ sim,
                                                              int8_t *__restrict__ xq, float *__restrict__ scale,
                                                              const float *__restrict__ simthr, int H, int N, int nb) {
-  constexpr int TPR = D / 8;
-  constexpr int RPP = 256 / TPR;
-  constexpr int NP = BS / RPP;
+  constexpr int ROWS = 128;           // rows per workgroup
+  constexpr int SUB = ROWS / BS;      // blocks per workgroup
+  constexpr int TPR = D / 8;          // lanes per row (16 B each)
+  constexpr int RPP = 256 / TPR;      // rows per pass of the workgroup
+  constexpr int NPT = ROWS / RPP;     // passes (rows per thread)
+  constexpr int NP = BS / RPP;        // passes per block
+  constexpr int WPS = D / 64;         // wavefronts that hold one block's columns in the tail (thread = block * D + column)
+  static_assert(BS == 64 || BS == 128, "block sizes of the operators");
+  static_assert(RPP <= BS && SUB * D <= 256, "thread <-> (block, column) mapping of the tail");
   // magnitude patterns (sign bit cleared) order like the magnitudes, for both 16-bit formats
   constexpr uint32_t ABS2 = 0x7fff7fffu;
   constexpr uint32_t INF16 = DT == 1 ? 0x7f80u : 0x7c00u;
   // "every element of the row is tiny": bfloat16 below 2^-63 (both top exponent bits clear), binary16 zero
   constexpr uint32_t TINY2 = DT == 1 ? 0x60006000u : 0x7fff7fffu;
-  const int blk = blockIdx.x, bh = blockIdx.y;
+  const int bh = blockIdx.y;
   const int tid = threadIdx.x, c = tid % TPR, r = tid / TPR;
-  const int row_base = blk * BS;
-  const int rows_valid = min(BS, N - row_base);
-  const bool partial = rows_valid < BS;          // workgroup-uniform: only the last block of a head
+  const int row_base = blockIdx.x * ROWS;
+  const int rows_here = min(ROWS, N - row_base);          // >= 1
+  const bool partial = rows_here < ROWS;                  // workgroup-uniform: only the last workgroup of a head
+  const int blk0 = blockIdx.x * SUB;
+  auto rows_valid_of = [&](int sb) { return max(0, min(BS, rows_here - sb * BS)); };
   const uint16_t *xb = x + (size_t)(bh / H) * xs.sb + (size_t)(bh % H) * xs.sh + (size_t)row_base * xs.sn + c * 8;
 
   float kmf[8];
@@ -177,22 +188,22 @@ __global__ __launch_bounds__(256) void pool_sim_quant_kernel(const uint16_t *__r
     unpack2<DT>(v.w, kmf[6], kmf[7]);
   }
 
-  // all loads of the thread are issued before the first use (rows beyond the block's end re-read its last row and
-  // are zeroed afterwards: no load sits behind a branch)
-  uint32_t w[NP][4];
+  // all loads of the thread are issued before the first use (rows beyond the end re-read the last row and are zeroed
+  // afterwards: no load sits behind a branch)
+  uint32_t w[NPT][4];
   {
-    uint4 raw[NP];
+    uint4 raw[NPT];
 #pragma unroll
-    for (int p = 0; p < NP; p++) raw[p] = *(const uint4 *)(xb + (size_t)min(r + p * RPP, rows_valid - 1) * xs.sn);
+    for (int p = 0; p < NPT; p++) raw[p] = *(const uint4 *)(xb + (size_t)min(r + p * RPP, rows_here - 1) * xs.sn);
 #pragma unroll
-    for (int p = 0; p < NP; p++) { w[p][0] = raw[p].x; w[p][1] = raw[p].y; w[p][2] = raw[p].z; w[p][3] = raw[p].w; }
+    for (int p = 0; p < NPT; p++) { w[p][0] = raw[p].x; w[p][1] = raw[p].y; w[p][2] = raw[p].z; w[p][3] = raw[p].w; }
   }
   if constexpr (HAS_MEAN) {
     // (k - km) rounded once to the input dtype (utils.py:184-188).  The binary32 difference of two 16-bit floats is
     // either exact or nowhere near a rounding tie of the 16-bit format, so rounding it to nearest even equals rounding
     // the exact difference.  The tile is kept as the rounded 16-bit patterns.
 #pragma unroll
-    for (int p = 0; p < NP; p++)
+    for (int p = 0; p < NPT; p++)
 #pragma unroll
       for (int j = 0; j < 4; j++) {
         float f0, f1;
@@ -202,50 +213,61 @@ __global__ __launch_bounds__(256) void pool_sim_quant_kernel(const uint16_t *__r
   }
   if (partial) {                                  // masked rows are zero (utils.py:188)
 #pragma unroll
-    for (int p = 0; p < NP; p++)
-      if (r + p * RPP >= rows_valid) { w[p][0] = 0; w[p][1] = 0; w[p][2] = 0; w[p][3] = 0; }
+    for (int p = 0; p < NPT; p++)
+      if (r + p * RPP >= rows_here) { w[p][0] = 0; w[p][1] = 0; w[p][2] = 0; w[p][3] = 0; }
   }
 
-  // largest magnitude of the thread's elements (as a 16-bit pattern) and, per row, whether all of them are tiny
-  uint32_t m2 = 0, tiny_rows = 0;
+  // largest magnitude of the thread's elements per block (as 16-bit patterns: block 0 in the low half, block 1 in the
+  // high half) and, per row, whether all of the thread's elements are tiny
+  uint32_t m_thread = 0, tiny_rows = 0;
 #pragma unroll
-  for (int p = 0; p < NP; p++) {
-    const uint32_t rm = pk_max_u16(pk_max_u16(w[p][0] & ABS2, w[p][1] & ABS2), pk_max_u16(w[p][2] & ABS2, w[p][3] & ABS2));
-    m2 = pk_max_u16(m2, rm);
-    if constexpr (WITH_POOL) tiny_rows |= ((rm & TINY2) == 0 ? 1u : 0u) << p;
+  for (int sb = 0; sb < SUB; sb++) {
+    uint32_t m2 = 0;
+#pragma unroll
+    for (int p = sb * NP; p < (sb + 1) * NP; p++) {
+      const uint32_t rm = pk_max_u16(pk_max_u16(w[p][0] & ABS2, w[p][1] & ABS2), pk_max_u16(w[p][2] & ABS2, w[p][3] & ABS2));
+      m2 = pk_max_u16(m2, rm);
+      if constexpr (WITH_POOL) tiny_rows |= ((rm & TINY2) == 0 ? 1u : 0u) << p;
+    }
+    m_thread |= max(m2 & 0xffffu, m2 >> 16) << (16 * sb);
   }
-  const uint32_t m_thread = max(m2 & 0xffffu, m2 >> 16);
-  __shared__ uint32_t s_wmax[4];
+  __shared__ uint32_t s_wmax[4], s_wbad[4];
   __shared__ long long s_wg[4];
   {
-    const uint32_t mw = wave_max_u32(m_thread);
+    uint32_t mw = m_thread;                       // both blocks' maxima reduced together
+#pragma unroll
+    for (int o = 32; o >= 1; o >>= 1) mw = pk_max_u16(mw, (uint32_t)__shfl_xor((int)mw, o, SPG_WAVE));
     if ((tid & 63) == 0) s_wmax[tid >> 6] = mw;
   }
 
   if constexpr (WITH_POOL) {
-    __shared__ double s_col[RPP][D];
-    __shared__ double s_xh[RPP][D];
-    double colsum[8];
-#pragma unroll
-    for (int e = 0; e < 8; e++) colsum[e] = 0.0;
+    // column sums of all blocks of the workgroup, one row group per line; used for the pooled mean first and, with a
+    // non-negative similarity threshold, for the normalised rows afterwards
+    __shared__ double s_red[SUB][RPP][D];
     // column sums for the pooled mean: binary64, exact
 #pragma unroll
-    for (int p = 0; p < NP; p++)
+    for (int sb = 0; sb < SUB; sb++) {
+      double colsum[8];
 #pragma unroll
-      for (int j = 0; j < 4; j++) {
-        float f0, f1;
-        forget(w[p][j]);
-        unpack2<DT>(w[p][j], f0, f1);
-        colsum[2 * j] += (double)f0;
-        colsum[2 * j + 1] += (double)f1;
-      }
+      for (int e = 0; e < 8; e++) colsum[e] = 0.0;
 #pragma unroll
-    for (int e = 0; e < 8; e++) s_col[r][c * 8 + e] = colsum[e];
+      for (int p = sb * NP; p < (sb + 1) * NP; p++)
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+          float f0, f1;
+          forget(w[p][j]);
+          unpack2<DT>(w[p][j], f0, f1);
+          colsum[2 * j] += (double)f0;
+          colsum[2 * j + 1] += (double)f1;
+        }
+#pragma unroll
+      for (int e = 0; e < 8; e++) s_red[sb][r][c * 8 + e] = colsum[e];
+    }
 
-    // row norms: the TPR lanes of a row group all need sqrt(sum of squares) and its reciprocal for each of their NP
-    // rows.  Both are computed ONCE per NP rows - lane c of the group takes row c % NP - and handed round with lane
-    // reads, instead of NP times in every lane.
-    static_assert(NP <= TPR, "one lane of the row group per row");
+    // row norms: the TPR lanes of a row group all need sqrt(sum of squares) and its reciprocal for each of their NPT
+    // rows.  Both are computed ONCE per NPT rows - lane c of the group takes row c % NPT - and handed round with lane
+    // reads, instead of NPT times in every lane.
+    static_assert(NPT <= TPR, "one lane of the row group per row");
     // A NEGATIVE similarity threshold (the top-k operators' default, -0.1) decides the flag without the normalised rows:
     // the statistic is ||sum of x_hat||^2 / rows^2 >= 0 > threshold whenever every x_hat is finite.  x_hat = x / norm is
     // non-finite exactly for rows with norm == 0 (all-zero rows such as the padding of a partial block, or rows too
@@ -255,18 +277,20 @@ __global__ __launch_bounds__(256) void pool_sim_quant_kernel(const uint16_t *__r
     // in which every element is smaller (all-zero rows, the padding of a partial block, bfloat16 values near the bottom
     // of the range) are decided by the exact sums below.
     const bool sim_trivial = simthr[bh % H] < 0.f;     // workgroup-uniform
-    int bad_rows = 0;
+    uint32_t bad = 0;                                  // bit sb: block sb holds a non-finite x_hat
     float ssf_mine = 0.f;
     bool need_norms = true;                            // wavefront-uniform
     if (sim_trivial) {
-      bad_rows |= m_thread >= INF16 ? 1 : 0;          // inf or NaN anywhere (overflowing squares of finite values are harmless: x / inf = 0)
+#pragma unroll
+      for (int sb = 0; sb < SUB; sb++)                 // inf or NaN anywhere (overflowing squares of finite values are harmless: x / inf = 0)
+        bad |= (((m_thread >> (16 * sb)) & 0xffffu) >= INF16 ? 1u : 0u) << sb;
       tiny_rows = group_and_u32<TPR>(tiny_rows);      // rows tiny in every lane of their group
       need_norms = __any(tiny_rows != 0);             // rare
     }
     if (need_norms) {
       // sum of squares of every row (exact in binary64), rounded to binary32 like the reference's (utils.py:194)
 #pragma unroll
-      for (int p = 0; p < NP; p++) {
+      for (int p = 0; p < NPT; p++) {
         double ss = 0.0;
 #pragma unroll
         for (int j = 0; j < 4; j++) {
@@ -279,103 +303,134 @@ __global__ __launch_bounds__(256) void pool_sim_quant_kernel(const uint16_t *__r
         }
         ss = group_sum_f64<TPR>(ss);                 // the TPR lanes of this row
         const float ssf = (float)ss;
-        ssf_mine = (c % NP == p) ? ssf : ssf_mine;
-        if (sim_trivial) bad_rows |= (ssf == 0.f) ? 1 : 0;
+        ssf_mine = (c % NPT == p) ? ssf : ssf_mine;
+        if (sim_trivial) bad |= ((ssf == 0.f) ? 1u : 0u) << (p / NP);
       }
     }
+    __syncthreads();
+    // tail: thread = block * D + column
+    const int t_sb = tid / D, t_col = tid % D;
+    const bool t_on = tid < SUB * D;
+    const int t_rows = rows_valid_of(t_sb);
+    if (t_on && t_rows > 0) {
+      double s = 0.0;
+      for (int i = 0; i < RPP; i++) s += s_red[t_sb][i][t_col];
+      // full blocks: the row count is a power of two, so the product with its reciprocal is the exact quotient
+      const double mean = t_rows == BS ? s * (1.0 / BS) : s / (double)t_rows;
+      pool[((size_t)bh * nb + blk0 + t_sb) * D + t_col] = f64_to_elem<DT>(mean);
+    }
+    long long g = 0;
     if (!sim_trivial) {
-      double colxh[8];
-#pragma unroll
-      for (int e = 0; e < 8; e++) colxh[e] = 0.0;
+      __syncthreads();                                // s_red is reused
       const float norm_mine = sqrtf(ssf_mine);
       const float rn_mine = rcp_safe(norm_mine) ? exact_rcp(norm_mine) : 0.f;
       const int group_lane0 = (tid & 63) & ~(TPR - 1);
 #pragma unroll
-      for (int p = 0; p < NP; p++) {
-        const float norm = __shfl(norm_mine, group_lane0 + p, SPG_WAVE);
-        const float rn = __shfl(rn_mine, group_lane0 + p, SPG_WAVE);
-        const bool fast = rcp_safe(norm);
+      for (int sb = 0; sb < SUB; sb++) {
+        double colxh[8];
 #pragma unroll
-        for (int j = 0; j < 4; j++) {
-          float f0, f1;
-          forget(w[p][j]);
-          unpack2<DT>(w[p][j], f0, f1);
-          // 0/0 -> NaN for all-zero (masked) rows on the slow branch
-          const _Float16 h0 = (_Float16)(fast ? div_by(f0, norm, rn) : f0 / norm);
-          const _Float16 h1 = (_Float16)(fast ? div_by(f1, norm, rn) : f1 / norm);
-          colxh[2 * j] += (double)(float)h0;          // fp16 values: integer multiples of 2^-24, sums are exact
-          colxh[2 * j + 1] += (double)(float)h1;
+        for (int e = 0; e < 8; e++) colxh[e] = 0.0;
+#pragma unroll
+        for (int p = sb * NP; p < (sb + 1) * NP; p++) {
+          const float norm = __shfl(norm_mine, group_lane0 + p, SPG_WAVE);
+          const float rn = __shfl(rn_mine, group_lane0 + p, SPG_WAVE);
+          const bool fast = rcp_safe(norm);
+#pragma unroll
+          for (int j = 0; j < 4; j++) {
+            float f0, f1;
+            forget(w[p][j]);
+            unpack2<DT>(w[p][j], f0, f1);
+            // the slow branch gives 0/0 = NaN for all-zero (masked) rows
+            const _Float16 h0 = (_Float16)(fast ? div_by(f0, norm, rn) : f0 / norm);
+            const _Float16 h1 = (_Float16)(fast ? div_by(f1, norm, rn) : f1 / norm);
+            colxh[2 * j] += (double)(float)h0;        // fp16 values: integer multiples of 2^-24, sums are exact
+            colxh[2 * j + 1] += (double)(float)h1;
+          }
+        }
+#pragma unroll
+        for (int e = 0; e < 8; e++) s_red[sb][r][c * 8 + e] = colxh[e];
+      }
+      __syncthreads();
+      if (t_on) {
+        double sx = 0.0;
+        for (int i = 0; i < RPP; i++) sx += s_red[t_sb][i][t_col];
+        if (__builtin_isfinite(sx)) {
+          const long long si = (long long)(sx * 16777216.0);   // exact integer
+          g = si * si;
+        } else {
+          bad |= 1u << t_sb;                          // a NaN/inf x_hat anywhere in the column
         }
       }
 #pragma unroll
-      for (int e = 0; e < 8; e++) s_xh[r][c * 8 + e] = colxh[e];
+      for (int o = 32; o >= 1; o >>= 1) g += shfl_xor_i64(g, o);
+      if ((tid & 63) == 0) s_wg[tid >> 6] = g;
+    }
+    // bit sb of any_bad: some thread saw a non-finite x_hat in block sb (one flag word per wavefront, combined below)
+    {
+      uint32_t wb = 0;
+#pragma unroll
+      for (int sb = 0; sb < SUB; sb++) wb |= (__any((bad >> sb) & 1u) ? 1u : 0u) << sb;
+      if ((tid & 63) == 0) s_wbad[tid >> 6] = wb;
     }
     __syncthreads();
-    long long g = 0;
-    int bad = bad_rows;
-    if (tid < D) {
-      double s = 0.0;
-      for (int i = 0; i < RPP; i++) s += s_col[i][tid];
-      pool[((size_t)bh * nb + blk) * D + tid] = f64_to_elem<DT>(s / (double)rows_valid);
-    }
-    if (!sim_trivial && tid < D) {
-      double sx = 0.0;
-      for (int i = 0; i < RPP; i++) sx += s_xh[i][tid];
-      if (__builtin_isfinite(sx)) {
-        const long long si = (long long)(sx * 16777216.0);   // exact integer
-        g = si * si;
-      } else {
-        bad = 1;                                    // a NaN/inf x_hat anywhere in the column
+    const uint32_t any_bad = s_wbad[0] | s_wbad[1] | s_wbad[2] | s_wbad[3];
+    if (tid < SUB && rows_valid_of(tid) > 0) {
+      const int rv = rows_valid_of(tid);
+      bool similar = sim_trivial;
+      if (!sim_trivial) {
+        long long gt = 0;                             // = sum(gram) * 2^48, exact
+        for (int i = 0; i < WPS; i++) gt += s_wg[tid * WPS + i];
+        const double thr = (double)simthr[bh % H] * (double)(rv * rv) * 281474976710656.0;
+        similar = (double)gt > thr;
       }
-    }
-#pragma unroll
-    for (int o = 32; o >= 1; o >>= 1) g += shfl_xor_i64(g, o);
-    if ((tid & 63) == 0) s_wg[tid >> 6] = g;
-    const int any_bad = __syncthreads_or(bad);
-    if (tid == 0) {
-      const long long gt = s_wg[0] + s_wg[1] + s_wg[2] + s_wg[3];   // = sum(gram) * 2^48, exact
-      const double thr = (double)simthr[bh % H] * (double)(rows_valid * rows_valid) * 281474976710656.0;
-      sim[(size_t)bh * nb + blk] = (!any_bad && (sim_trivial || (double)gt > thr)) ? 1 : 0;
+      sim[(size_t)bh * nb + blk0 + tid] = (!((any_bad >> tid) & 1u) && similar) ? 1 : 0;
     }
   } else {
     __syncthreads();
   }
 
-  const uint32_t m_blk = max(max(s_wmax[0], s_wmax[1]), max(s_wmax[2], s_wmax[3]));
-  const float amax = elem_to_f32<DT>((uint16_t)m_blk);
-  const float s = amax / 127.0f + 1e-7f;
+  const uint32_t m_all = pk_max_u16(pk_max_u16(s_wmax[0], s_wmax[1]), pk_max_u16(s_wmax[2], s_wmax[3]));
   int8_t *qb = xq + ((size_t)bh * N + row_base) * D + c * 8;
-  auto quantise = [&](auto divide) {
 #pragma unroll
-    for (int p = 0; p < NP; p++) {
-      const int row = r + p * RPP;
-      if (!partial || row < rows_valid) {
-        uint32_t pk[2] = {0, 0};
+  for (int sb = 0; sb < SUB; sb++) {
+    if (rows_valid_of(sb) <= 0) break;                  // workgroup-uniform
+    const float amax = elem_to_f32<DT>((uint16_t)(m_all >> (16 * sb)));
+    const float s = amax / 127.0f + 1e-7f;
+    auto quantise = [&](auto divide, auto check_rows) {
 #pragma unroll
-        for (int j = 0; j < 4; j++) {
-          float f[2];
-          forget(w[p][j]);
-          unpack2<DT>(w[p][j], f[0], f[1]);
+      for (int p = sb * NP; p < (sb + 1) * NP; p++) {
+        const int row = r + p * RPP;
+        if (!decltype(check_rows)::value || row < rows_here) {
+          uint32_t pk[2] = {0, 0};
 #pragma unroll
-          for (int h = 0; h < 2; h++) {
-            float y = divide(f[h]);
-            y = y + __builtin_copysignf(0.5f, y);   // +0.5 for y >= 0 (a -0 quotient truncates to 0 either way)
-            const int q = (int)y;   // truncation toward zero
-            const int e = 2 * j + h;
-            pk[e >> 2] |= ((uint32_t)q & 0xffu) << (8 * (e & 3));
+          for (int j = 0; j < 4; j++) {
+            float f[2];
+            forget(w[p][j]);
+            unpack2<DT>(w[p][j], f[0], f[1]);
+#pragma unroll
+            for (int h = 0; h < 2; h++) {
+              float y = divide(f[h]);
+              y = y + __builtin_copysignf(0.5f, y);   // +0.5 for y >= 0 (a -0 quotient truncates to 0 either way)
+              const int q = (int)y;   // truncation toward zero
+              const int e = 2 * j + h;
+              pk[e >> 2] |= ((uint32_t)q & 0xffu) << (8 * (e & 3));
+            }
           }
+          *(uint2 *)(qb + (size_t)row * D) = make_uint2(pk[0], pk[1]);
         }
-        *(uint2 *)(qb + (size_t)row * D) = make_uint2(pk[0], pk[1]);
       }
+    };
+    if (rcp_safe(s) && !partial) {         // workgroup-uniform; the common case carries no row test
+      const float rs = exact_rcp(s);
+      quantise([&](float v) { return div_by(v, s, rs); }, std::false_type{});
+    } else if (rcp_safe(s)) {
+      const float rs = exact_rcp(s);
+      quantise([&](float v) { return div_by(v, s, rs); }, std::true_type{});
+    } else {
+      quantise([&](float v) { return v / s; }, std::true_type{});
     }
-  };
-  if (rcp_safe(s)) {                     // workgroup-uniform
-    const float rs = exact_rcp(s);
-    quantise([&](float v) { return div_by(v, s, rs); });
-  } else {
-    quantise([&](float v) { return v / s; });
+    if (tid == 0) scale[(size_t)bh * nb + blk0 + sb] = s;
   }
-  if (tid == 0) scale[(size_t)bh * nb + blk] = s;
 }
 
 // =============================================================================================
@@ -1008,7 +1063,7 @@ template <int BS, int D, int DT>
 static void launch_psq3(const void *x, Strides xs, const void *km, void *pool, uint8_t *sim, int8_t *xq, float *scale,
                         const float *thr, int B, int H, int N, hipStream_t st) {
   const int nb = (N + BS - 1) / BS;
-  const dim3 grid(nb, B * H);
+  const dim3 grid((N + 127) / 128, B * H);      // one workgroup per 128 rows: one or two blocks
   const uint16_t *xp = (const uint16_t *)x, *kp = (const uint16_t *)km;
   uint16_t *pp = (uint16_t *)pool;
   if (pool != nullptr) {
