@@ -33,19 +33,24 @@ __global__ __launch_bounds__(256) void v_absmax_kernel(const uint16_t *__restric
   const int row0 = chunk * rows_per_chunk;
   const int row1 = min(N, row0 + rows_per_chunk);
   const uint16_t *base = v + (size_t)(bh / H) * vs.sb + (size_t)(bh % H) * vs.sh + c * 8;
-  float m[8];
-#pragma unroll
-  for (int e = 0; e < 8; e++) m[e] = 0.f;
-#pragma unroll 4
+  // The cast to fp16 is monotonic in the magnitude, so the largest |fp16(v)| is the cast of the largest |v|: the maximum
+  // is taken on the 16-bit magnitude patterns (which order like the magnitudes), two per instruction, and only the
+  // result is converted.
+  typedef unsigned short u16x2_t __attribute__((ext_vector_type(2)));
+  uint32_t mp[4] = {0, 0, 0, 0};
+#pragma unroll 8
   for (int row = row0 + r; row < row1; row += RPP) {
     const uint4 q = *(const uint4 *)(base + (size_t)row * vs.sn);
     const uint32_t w[4] = {q.x, q.y, q.z, q.w};
 #pragma unroll
-    for (int e = 0; e < 8; e++) {
-      const uint16_t b = (uint16_t)((e & 1) ? (w[e >> 1] >> 16) : (w[e >> 1] & 0xffffu));
-      m[e] = fmaxf(m[e], fabsf(elem_to_f16_f32<DT>(b)));
-    }
+    for (int j = 0; j < 4; j++)
+      mp[j] = __builtin_bit_cast(uint32_t, __builtin_elementwise_max(__builtin_bit_cast(u16x2_t, mp[j]),
+                                                                      __builtin_bit_cast(u16x2_t, w[j] & 0x7fff7fffu)));
   }
+  float m[8];
+#pragma unroll
+  for (int e = 0; e < 8; e++)
+    m[e] = elem_to_f16_f32<DT>((uint16_t)((e & 1) ? (mp[e >> 1] >> 16) : (mp[e >> 1] & 0xffffu)));
   __shared__ float sm[RPP][D];
 #pragma unroll
   for (int e = 0; e < 8; e++) sm[r][c * 8 + e] = m[e];
