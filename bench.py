@@ -273,7 +273,7 @@ def main():
 
     if not args.no_dense:
         qh, kh, vh = q.to(torch.float16), k.to(torch.float16), v.to(torch.float16)
-        vt = _lib.v_tiles_f16(vh)
+        vt = _lib.v_tiles_f16_swizzled(vh)
         oh = torch.empty_like(qh)
         sc = 1.0 / D ** 0.5
         for _ in range(max(1, args.warmup)):

@@ -152,7 +152,8 @@ int spg_block_sparse_attn_f16v(const int8_t *q8, const int8_t *k8, const void *v
 
 /* ---- measurement comparator: dense FP16 flash attention on MFMA (no counterpart in the reference;
  * the "dense FP16 attention kernel built in the same run" the speed-up is quoted against).
- * q,k,out (B,H,N,D) fp16; vt = V transposed per 64-key block, (B,H,ceil(N/64),D,64) fp16, zero-padded. */
+ * q,k,out (B,H,N,D) fp16; vt = the fp16 V^T tiles spg_v_tiles_f16 writes, (B,H,ceil(N/64),D,64), chunk-swizzled,
+ * zero beyond N. */
 int spg_dense_attn_f16(const void *q, const void *k, const void *vt, void *out, int B, int H, int N, int D,
                        float sm_scale, int is_causal, void *stream);
 

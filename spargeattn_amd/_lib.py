@@ -295,17 +295,8 @@ def block_sparse_attn_f16v(q8, k8, vt, out, lut, valid, pvthreshd, q_scale, k_sc
     return pvc
 
 
-def v_tiles_f16(v):
-    """(B,H,N,D) fp16 -> zero-padded (B,H,nk,D,64) tiles, the V^T layout the dense comparator reads."""
-    B, H, N, D = v.shape
-    nk = (N + 63) // 64
-    if nk * 64 != N:
-        v = torch.nn.functional.pad(v, (0, 0, 0, nk * 64 - N))
-    return v.view(B, H, nk, 64, D).transpose(-1, -2).contiguous()
-
-
 def dense_attn_f16(q, k, vt, sm_scale, is_causal=False, out=None):
-    """Dense fp16 flash attention (measurement comparator).  vt = v_tiles_f16(v)."""
+    """Dense fp16 flash attention (measurement comparator).  vt = v_tiles_f16_swizzled(v)."""
     _dev(q, k, vt)
     assert q.dtype == k.dtype == vt.dtype == torch.float16
     B, H, N, D = q.shape

@@ -27,12 +27,12 @@
 //  * workgroup ids are remapped so that one XCD (one L2) works on one head at a time, heaviest rows first.
 #include "common.h"
 #include "launch.h"
+#include "lds_asm.h"
 
 #include <type_traits>
 
 namespace spg {
 
-typedef int v4i __attribute__((ext_vector_type(4)));
 typedef int v8i __attribute__((ext_vector_type(8)));
 typedef int v8i_a16 __attribute__((ext_vector_type(8), aligned(16)));
 typedef int v16i __attribute__((ext_vector_type(16)));
@@ -59,25 +59,6 @@ struct AttnParams {
   int total_wg, wg_per_xcd;
 };
 
-// LDS tile reads are issued through inline asm with explicit waits.  Left to the compiler, every LDS read would be
-// ordered after ALL outstanding direct-to-LDS loads of the ring (s_waitcnt vmcnt(0)), which serialises the prefetch
-// of block it+2 with the compute of block it.  The ring's own protocol (vmcnt(0) + barrier before a slot is read)
-// is what guarantees correctness.
-template <int OFF0, int OFF1>
-__device__ __forceinline__ void lds_read_2x128(v4i &a, v4i &b, uint32_t addr) {
-  asm volatile("ds_read_b128 %0, %2 offset:%3\n\tds_read_b128 %1, %2 offset:%4"
-               : "=&v"(a), "=&v"(b)
-               : "v"(addr), "n"(OFF0), "n"(OFF1)
-               : "memory");
-}
-// two reads at the same immediate offset from two addresses (the two key chunks of a V^T row)
-template <int OFF>
-__device__ __forceinline__ void lds_read_pair(v4i &a, v4i &b, uint32_t addr_a, uint32_t addr_b) {
-  asm volatile("ds_read_b128 %0, %2 offset:%4\n\tds_read_b128 %1, %3 offset:%4"
-               : "=&v"(a), "=&v"(b)
-               : "v"(addr_a), "v"(addr_b), "n"(OFF)
-               : "memory");
-}
 // v_max_f32 as one instruction: fmaxf() on a value the compiler cannot prove to be a quiet number (a loop-carried
 // maximum, the output of a lane exchange) costs a canonicalising self-maximum per operand first.  The operands here are
 // products and maxima of finite numbers.
@@ -92,12 +73,6 @@ __device__ __forceinline__ float half_swap_max_raw(float v) {
   asm("s_nop 0\n\tv_max_f32 %0, %1, %2" : "=v"(r) : "v"(lo), "v"(hi));   // one idle state behind the lane exchange
   return r;
 }
-// wait for all outstanding LDS reads; the operands tie the wait to the registers it makes valid
-__device__ __forceinline__ void lds_wait4(v4i &a, v4i &b, v4i &c, v4i &d) {
-  asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(a), "+v"(b), "+v"(c), "+v"(d));
-}
-__device__ __forceinline__ void lds_wait2(v4i &a, v4i &b) { asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(a), "+v"(b)); }
-
 // e4m3 pack of the probabilities.  v_cvt_pk_fp8_f32 returns NaN (0x7f) for |x| > 464 unless MODE.FP16_OVFL is set, in
 // which case finite values clamp to +-448 like the reference's cvt.rn.satfinite.e4m3x2.f32 (csrc/numeric_conversion.cuh:48-63);
 // the bit is set once per wavefront, costs nothing per element and affects no other instruction this kernel depends on

@@ -1,8 +1,15 @@
 // Dense FP16 flash attention on gfx950 MFMA: the comparator the sparse path's speed-up is quoted against.
-// Same skeleton as attn.hip (transposed products, one query column per lane, double-buffered LDS tiles, XCD-aware
-// workgroup order) with v_mfma_f32_32x32x16_f16 for both products and fp16 P.  Not part of the reference.
+// Same skeleton as attn.hip: transposed products (one query column per lane), K rows permuted so that the 32 scores of
+// a lane are 32 consecutive keys, K / V^T tiles brought from HBM/L2 straight into LDS (global_load_lds, no register
+// staging) through a two-slot ring with ONE barrier per block, unpadded LDS tiles with XOR-swizzled 16-byte chunks, LDS
+// operand reads through inline asm with their own waits, XCD-aware workgroup order; v_mfma_f32_32x32x16_f16 for both
+// products and fp16 P.  Not part of the reference.
+//
+// V comes as the fp16 V^T tiles of spg_v_tiles_f16: [nk][D][64] fp16, the eight 8-key chunks of a 128-byte row stored
+// at slot = chunk ^ ((d >> 1) & 7), zero beyond N.
 #include "common.h"
 #include "launch.h"
+#include "lds_asm.h"
 
 namespace spg {
 
@@ -18,23 +25,34 @@ struct DenseParams {
   int total_wg, wg_per_xcd;
 };
 
+// K tile row = key (2 D bytes = D/8 chunks of 16 bytes).  A half-wavefront reads the K operand from key rows
+// {0..15} u {32..47} (+16 for the second key tile) at one chunk index; the swizzle spreads those 32 rows evenly over the
+// sixteen 16-byte slots of a 256-byte LDS line (two lanes per slot).
+template <int D>
+__device__ __forceinline__ uint32_t dense_k_swz(uint32_t row) {
+  if constexpr (D == 128) return row & 15u;          // one row per line: 16 chunks
+  else return (row >> 1) & 7u;                       // two rows per line: bit 0 of the row is already a slot bit
+}
+
 template <int D>
 __global__ __launch_bounds__(256, 2) void dense_attn_f16_kernel(const DenseParams p) {
   constexpr int KS = D / 16;          // k-steps of QK^T
   constexpr int NDT = D / 32;         // output channel tiles
-  constexpr int KSTR = D * 2 + 16;    // bytes per K row in LDS
-  constexpr int VSTR = 64 * 2 + 16;   // bytes per V^T row in LDS
-  constexpr int CH = D / 32;          // 16-byte chunks per thread per tile (64*D*2/16/256)
-  extern __shared__ __align__(16) unsigned char smem[];
-  auto sKp = [&](int b) -> unsigned char * { return smem + b * (64 * KSTR); };
-  auto sVp = [&](int b) -> unsigned char * { return smem + 2 * 64 * KSTR + b * (D * VSTR); };
+  constexpr int TILE = 64 * D * 2;    // bytes of one K tile and of one V^T tile
+  constexpr int CPR = D / 8;          // 16-byte chunks per K row
+  constexpr int WL = TILE / 4096;     // global_load_lds instructions per wavefront per tile
+  constexpr int NBUF = 2;
+  __shared__ __align__(1024) unsigned char smem[NBUF * 2 * TILE];   // K ring | V^T ring
+  const uint32_t lds_k0 = (uint32_t)(size_t)(__attribute__((address_space(3))) unsigned char *)smem;
+  const uint32_t lds_v0 = lds_k0 + NBUF * TILE;
 
   const int w = blockIdx.x;
   const int L = (w & 7) * p.wg_per_xcd + (w >> 3);
   if (L >= p.total_wg) return;
   const int bh = L / p.nq;
   const int qb = p.nq - 1 - (L % p.nq);
-  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, r = lane & 31, hh = lane >> 5;
+  const int tid = threadIdx.x, lane = tid & 63, r = lane & 31, hh = lane >> 5;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int N = p.N;
   const int q_row = qb * 128 + wave * 32 + r;
   const int nblk = p.is_causal ? min(p.nk, 2 * (qb + 1)) : p.nk;
@@ -46,36 +64,59 @@ __global__ __launch_bounds__(256, 2) void dense_attn_f16_kernel(const DenseParam
     if (q_row < N) t = *(const uint4 *)(p.q + ((size_t)bh * N + q_row) * D + 16 * ks + 8 * hh);
     qreg[ks] = __builtin_bit_cast(v8h, t);
   }
-  const uint16_t *kbase = p.k + (size_t)bh * N * D;
-  const uint16_t *vbase = p.vt + (size_t)bh * p.nk * (size_t)(D * 64);
+  const unsigned char *kbase = (const unsigned char *)(p.k + (size_t)bh * N * D);
+  const unsigned char *vbase = (const unsigned char *)(p.vt + (size_t)bh * p.nk * (size_t)(D * 64));
   const float c = p.sm_scale_log2;
 
-  // staging registers for the next block's tiles (named scalars: an indexed array ends up in scratch memory)
-  uint4 kr0, kr1, kr2, kr3, vr0, vr1, vr2, vr3;
-  kr0 = kr1 = kr2 = kr3 = vr0 = vr1 = vr2 = vr3 = make_uint4(0, 0, 0, 0);
-#define SPG_FETCH1(U, KR, VR, BLK)                                                                       \
-  if constexpr (CH > U) {                                                                                \
-    const int ci = tid + 256 * U;                                                                        \
-    const int row = ci / (D / 8), col = ci % (D / 8);                                                    \
-    /* rows beyond N (last block only) are clamped to a valid row: their scores are masked below */      \
-    const int grow = min((BLK) * 64 + row, N - 1);                                                       \
-    KR = *(const uint4 *)(kbase + (size_t)grow * D + col * 8);                                           \
-    VR = *(const uint4 *)(vbase + (size_t)(BLK) * (D * 64) + (size_t)ci * 8);                            \
+  // ---- tile loader: wavefront w copies LDS bytes [1024 (WL w + u), +1024) of each tile, lane l the 16-byte chunk l.
+  // K: LDS chunk position pos <-> (row = pos / CPR, slot = pos % CPR) holds global chunk slot ^ swz(row); V^T tiles are
+  // stored swizzled in HBM and copied verbatim.  Rows beyond N (last block only) are clamped to row N - 1: their scores
+  // are masked below and their V rows are zero.
+  typedef __attribute__((address_space(3))) void *lds_ptr_t;
+  typedef const __attribute__((address_space(1))) void *glb_ptr_t;
+  uint32_t k_off[WL];
+#pragma unroll
+  for (int u = 0; u < WL; u++) {
+    const uint32_t pos = (uint32_t)(64 * (WL * wave + u) + lane);
+    const uint32_t row = pos / CPR, slot = pos % CPR;
+    k_off[u] = row * (D * 2) + ((slot ^ dense_k_swz<D>(row)) * 16u);
   }
-#define SPG_FETCH(BLK)                                                                                   \
-  { SPG_FETCH1(0, kr0, vr0, BLK) SPG_FETCH1(1, kr1, vr1, BLK) SPG_FETCH1(2, kr2, vr2, BLK) SPG_FETCH1(3, kr3, vr3, BLK) }
-#define SPG_STASH1(U, KR, VR, BUF)                                                                       \
-  if constexpr (CH > U) {                                                                                \
-    const int ci = tid + 256 * U;                                                                        \
-    *(uint4 *)(sKp(BUF) + (ci / (D / 8)) * KSTR + (ci % (D / 8)) * 16) = KR;                             \
-    *(uint4 *)(sVp(BUF) + (ci >> 3) * VSTR + (ci & 7) * 16) = VR;                                        \
-  }
-#define SPG_STASH(BUF)                                                                                   \
-  { SPG_STASH1(0, kr0, vr0, BUF) SPG_STASH1(1, kr1, vr1, BUF) SPG_STASH1(2, kr2, vr2, BUF) SPG_STASH1(3, kr3, vr3, BUF) }
+  const uint32_t v_off = (uint32_t)(WL * 1024 * wave + 16 * lane);
+  const int last_partial_blk = (N % 64) ? p.nk - 1 : -1;
+  auto load_tiles = [&](int blk, int slot) __attribute__((always_inline)) {
+    const unsigned char *kb = kbase + (size_t)blk * TILE;
+    const unsigned char *vb = vbase + (size_t)blk * TILE;
+    unsigned char *lk = smem + slot * TILE + WL * wave * 1024;
+    unsigned char *lv = smem + (NBUF + slot) * TILE + WL * wave * 1024;
+    if (blk != last_partial_blk) {
+#pragma unroll
+      for (int u = 0; u < WL; u++)
+        __builtin_amdgcn_global_load_lds((glb_ptr_t)(kb + k_off[u]), (lds_ptr_t)(lk + u * 1024), 16, 0, 0);
+    } else {
+      const uint32_t rows_ok = (uint32_t)(N - blk * 64);
+#pragma unroll
+      for (int u = 0; u < WL; u++) {
+        const uint32_t pos = (uint32_t)(64 * (WL * wave + u) + lane);
+        const uint32_t row = min(pos / CPR, rows_ok - 1), slot_ = pos % CPR;
+        const uint32_t ko = row * (D * 2) + ((slot_ ^ dense_k_swz<D>(pos / CPR)) * 16u);
+        __builtin_amdgcn_global_load_lds((glb_ptr_t)(kb + ko), (lds_ptr_t)(lk + u * 1024), 16, 0, 0);
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < WL; u++)
+      __builtin_amdgcn_global_load_lds((glb_ptr_t)(vb + v_off + u * 1024), (lds_ptr_t)(lv + u * 1024), 16, 0, 0);
+  };
 
-  // MFMA row i of key tile kt carries key 32*kt + 16*(i>>4) + 8*((i>>2)&1) + 4*((i>>3)&1) + (i&3):
-  // after S^T, the 8 registers [8n', 8n'+8) of a lane hold 8 consecutive keys 16*(2kt+n') + 8*half + (0..7).
-  const int krow0 = 16 * (r >> 4) + 8 * ((r >> 2) & 1) + 4 * ((r >> 3) & 1) + (r & 3);
+  // MFMA row i of key tile kt carries key 32*((i>>2)&1) + 16*kt + 4*(i>>3) + (i&3): after S^T, register e of tile kt in
+  // lane (r, hh) is key 32 hh + 16 kt + e, i.e. the lane's 32 scores are 32 consecutive keys.  Rows krow0 and krow0 + 16
+  // have the same swizzle, so tile 1's operand sits 16 rows after tile 0's.
+  const uint32_t krow0 = (uint32_t)(32 * ((r >> 2) & 1) + 4 * (r >> 3) + (r & 3));
+  const uint32_t ksw = dense_k_swz<D>(krow0);
+  uint32_t kaddr[KS];
+#pragma unroll
+  for (int ks = 0; ks < KS; ks++) kaddr[ks] = lds_k0 + krow0 * (D * 2) + ((((uint32_t)(2 * ks + hh)) ^ ksw) * 16u);
+  // V^T operand of key step s: chunk (4 hh + s) ^ ((r >> 1) & 7) of the 128-byte row r (+ 32 dt): va ^ (16 s)
+  const uint32_t va0 = lds_v0 + (uint32_t)(r * 128 + (((4 * hh) ^ ((r >> 1) & 7)) * 16));
 
   float m = -INFINITY, dsum = 0.f;
   v16f O[NDT];
@@ -84,40 +125,58 @@ __global__ __launch_bounds__(256, 2) void dense_attn_f16_kernel(const DenseParam
 #pragma unroll
     for (int e = 0; e < 16; e++) O[dt][e] = 0.f;
 
-  SPG_FETCH(0);
-  SPG_STASH(0);
-  int buf = 0;
+  load_tiles(0, 0);
+  __builtin_amdgcn_s_waitcnt(0x0F70);     // vmcnt(0)
+  __syncthreads();
+
+#pragma unroll 1
   for (int blk = 0; blk < nblk; blk++) {
-    __syncthreads();
-    v16f S[2];
+    const uint32_t so = (uint32_t)(blk & 1) * TILE;
+    // slot (blk+1)&1 was last read in iteration blk-1, which every wavefront has left (barrier at its end)
+    if (blk + 1 < nblk) load_tiles(blk + 1, (blk + 1) & 1);
+
+    // ---- S^T = K . Q^T: the reads of the second half of the k-steps are in flight while the first half multiplies
+    v16f S0, S1;
 #pragma unroll
-    for (int e = 0; e < 16; e++) { S[0][e] = 0.f; S[1][e] = 0.f; }
+    for (int e = 0; e < 16; e++) { S0[e] = 0.f; S1[e] = 0.f; }
+    {
+      constexpr int HK = KS / 2;
+      v4i a0[KS], a1[KS];
 #pragma unroll
-    for (int ks = 0; ks < KS; ks++) {
+      for (int ks = 0; ks < HK; ks++) lds_read_2x128<0, 16 * D * 2>(a0[ks], a1[ks], kaddr[ks] + so);
+      if constexpr (HK == 4) { lds_wait4(a0[0], a1[0], a0[1], a1[1]); lds_wait4(a0[2], a1[2], a0[3], a1[3]); }
+      else lds_wait4(a0[0], a1[0], a0[1], a1[1]);
 #pragma unroll
-      for (int kt = 0; kt < 2; kt++) {
-        const uint4 t = *(const uint4 *)(sKp(buf) + (krow0 + 32 * kt) * KSTR + (16 * ks + 8 * hh) * 2);
-        S[kt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(v8h, t), qreg[ks], S[kt], 0, 0, 0);
+      for (int ks = HK; ks < KS; ks++) lds_read_2x128<0, 16 * D * 2>(a0[ks], a1[ks], kaddr[ks] + so);
+#pragma unroll
+      for (int ks = 0; ks < HK; ks++) {
+        S0 = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(v8h, a0[ks]), qreg[ks], S0, 0, 0, 0);
+        S1 = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(v8h, a1[ks]), qreg[ks], S1, 0, 0, 0);
+      }
+      if constexpr (HK == 4) { lds_wait4(a0[4], a1[4], a0[5], a1[5]); lds_wait4(a0[6], a1[6], a0[7], a1[7]); }
+      else lds_wait4(a0[2], a1[2], a0[3], a1[3]);
+#pragma unroll
+      for (int ks = HK; ks < KS; ks++) {
+        S0 = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(v8h, a0[ks]), qreg[ks], S0, 0, 0, 0);
+        S1 = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(v8h, a1[ks]), qreg[ks], S1, 0, 0, 0);
       }
     }
-    const bool more = blk + 1 < nblk;
-    SPG_FETCH(more ? blk + 1 : blk);   // unconditional: keeps the staging registers out of scratch
 
-    // register e of tile kt <-> key 64*blk + 32*kt + 16*(e>>3) + 8*hh + (e&7)
+    // slot e of this lane is key 64 blk + 32 hh + e (e < 16: S0[e], else S1[e - 16])
     const bool edge = (p.is_causal && blk >= 2 * qb) || (blk == p.nk - 1);
-    float fm = -INFINITY;
+    float x[32];
 #pragma unroll
-    for (int kt = 0; kt < 2; kt++)
+    for (int e = 0; e < 32; e++) x[e] = e < 16 ? S0[e] : S1[e - 16];
+    if (edge) {
+      const int key0 = 64 * blk + 32 * hh;
+      int lim = N - 1 - key0;
+      if (p.is_causal) lim = min(lim, q_row - key0);
 #pragma unroll
-      for (int e = 0; e < 16; e++) {
-        float v = S[kt][e];
-        if (edge) {
-          const int key = 64 * blk + 32 * kt + 16 * (e >> 3) + 8 * hh + (e & 7);
-          if (key >= N || (p.is_causal && key > q_row)) v = -INFINITY;
-          S[kt][e] = v;
-        }
-        fm = fmaxf(fm, v);
-      }
+      for (int e = 0; e < 32; e++) x[e] = e > lim ? -INFINITY : x[e];
+    }
+    float fm = x[0];
+#pragma unroll
+    for (int e = 1; e < 32; e++) fm = fmaxf(fm, x[e]);
     fm = half_swap_max_f32(fm) * c;
     const float m_new = fmaxf(m, fm);
     const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
@@ -130,36 +189,57 @@ __global__ __launch_bounds__(256, 2) void dense_attn_f16_kernel(const DenseParam
 #pragma unroll
         for (int e = 0; e < 16; e++) O[dt][e] *= osc;
     }
-    v8h pb[4];
+#pragma unroll
+    for (int e = 0; e < 32; e++) x[e] = __builtin_fmaf(x[e], c, -m_use);
+#pragma unroll
+    for (int e = 0; e < 32; e++) x[e] = __builtin_amdgcn_exp2f(x[e]);
     float ps = 0.f;
 #pragma unroll
-    for (int kt = 0; kt < 2; kt++)
-#pragma unroll
-      for (int e = 0; e < 16; e += 2) {
-        const float p0 = __builtin_amdgcn_exp2f(__builtin_fmaf(S[kt][e], c, -m_use));
-        const float p1 = __builtin_amdgcn_exp2f(__builtin_fmaf(S[kt][e + 1], c, -m_use));
-        ps += p0 + p1;
-        const auto h2 = __builtin_amdgcn_cvt_pkrtz(p0, p1);      // two fp16 in one instruction
-        pb[2 * kt + (e >> 3)][e & 7] = (_Float16)h2[0];
-        pb[2 * kt + (e >> 3)][(e & 7) + 1] = (_Float16)h2[1];
-      }
+    for (int e = 0; e < 32; e++) ps += x[e];
     dsum += ps;
+    v8h pb[4];
 #pragma unroll
-    for (int n = 0; n < 4; n++) {
+    for (int s4 = 0; s4 < 4; s4++)
 #pragma unroll
-      for (int dt = 0; dt < NDT; dt++) {
-        const uint4 t = *(const uint4 *)(sVp(buf) + (32 * dt + r) * VSTR + (16 * n + 8 * hh) * 2);
-        O[dt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(v8h, t), pb[n], O[dt], 0, 0, 0);
+      for (int j = 0; j < 8; j += 2) {
+        const auto h2 = __builtin_amdgcn_cvt_pkrtz(x[8 * s4 + j], x[8 * s4 + j + 1]);   // two fp16 in one instruction
+        pb[s4][j] = (_Float16)h2[0];
+        pb[s4][j + 1] = (_Float16)h2[1];
       }
+
+    // ---- O^T += V^T . P^T: key steps 0,1 are read first; steps 2,3 are in flight while 0,1 multiply
+    {
+      const uint32_t va = va0 + so;
+      v4i t[4][NDT];
+#pragma unroll
+      for (int s4 = 0; s4 < 2; s4++) {
+        lds_read_2x128<0, 4096>(t[s4][0], t[s4][1], va ^ (uint32_t)(16 * s4));
+        if constexpr (NDT == 4) lds_read_2x128<8192, 12288>(t[s4][2], t[s4][3], va ^ (uint32_t)(16 * s4));
+      }
+      if constexpr (NDT == 4) { lds_wait4(t[0][0], t[0][1], t[0][2], t[0][3]); lds_wait4(t[1][0], t[1][1], t[1][2], t[1][3]); }
+      else { lds_wait4(t[0][0], t[0][1], t[1][0], t[1][1]); }
+#pragma unroll
+      for (int s4 = 2; s4 < 4; s4++) {
+        lds_read_2x128<0, 4096>(t[s4][0], t[s4][1], va ^ (uint32_t)(16 * s4));
+        if constexpr (NDT == 4) lds_read_2x128<8192, 12288>(t[s4][2], t[s4][3], va ^ (uint32_t)(16 * s4));
+      }
+#pragma unroll
+      for (int s4 = 0; s4 < 2; s4++)
+#pragma unroll
+        for (int dt = 0; dt < NDT; dt++)
+          O[dt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(v8h, t[s4][dt]), pb[s4], O[dt], 0, 0, 0);
+      if constexpr (NDT == 4) { lds_wait4(t[2][0], t[2][1], t[2][2], t[2][3]); lds_wait4(t[3][0], t[3][1], t[3][2], t[3][3]); }
+      else { lds_wait4(t[2][0], t[2][1], t[3][0], t[3][1]); }
+#pragma unroll
+      for (int s4 = 2; s4 < 4; s4++)
+#pragma unroll
+        for (int dt = 0; dt < NDT; dt++)
+          O[dt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(v8h, t[s4][dt]), pb[s4], O[dt], 0, 0, 0);
     }
-    SPG_STASH(buf ^ 1);                // buf^1 was last read before this iteration's barrier
-    buf ^= 1;
+    __builtin_amdgcn_s_waitcnt(0x0F70);   // this wavefront's share of block blk+1's tiles has landed in LDS
+    __syncthreads();                      // block blk+1's tiles are complete; every wavefront is done with block blk's
   }
 
-#undef SPG_FETCH
-#undef SPG_STASH
-#undef SPG_FETCH1
-#undef SPG_STASH1
   const float dtot = half_swap_sum_f32(dsum);
   const float inv = 1.0f / dtot;
   if (q_row < N) {
@@ -178,18 +258,6 @@ __global__ __launch_bounds__(256, 2) void dense_attn_f16_kernel(const DenseParam
   }
 }
 
-template <int D>
-static hipError_t launch_dense(const DenseParams &p, hipStream_t st) {
-  constexpr size_t lds = 2 * 64 * (D * 2 + 16) + 2 * D * (64 * 2 + 16);
-  auto kern = dense_attn_f16_kernel<D>;
-  if (lds > 48 * 1024) {
-    hipError_t e = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-    if (e != hipSuccess) return e;
-  }
-  kern<<<p.wg_per_xcd * 8, 256, lds, st>>>(p);
-  return hipGetLastError();
-}
-
 hipError_t launch_dense_attn_f16(const void *q, const void *k, const void *vt, void *out, int B, int H, int N, int D,
                                  float sm_scale, int is_causal, hipStream_t st) {
   DenseParams p;
@@ -199,7 +267,9 @@ hipError_t launch_dense_attn_f16(const void *q, const void *k, const void *vt, v
   p.is_causal = is_causal;
   p.total_wg = p.nq * H * B;
   p.wg_per_xcd = (p.total_wg + 7) / 8;
-  return D == 64 ? launch_dense<64>(p, st) : launch_dense<128>(p, st);
+  if (D == 64) dense_attn_f16_kernel<64><<<p.wg_per_xcd * 8, 256, 0, st>>>(p);
+  else dense_attn_f16_kernel<128><<<p.wg_per_xcd * 8, 256, 0, st>>>(p);
+  return hipGetLastError();
 }
 
 }  // namespace spg

@@ -218,7 +218,7 @@ def test_fp32_input_and_error_paths():
 def test_dense_f16_comparator(D, N, causal):
     B, H = 1, 2
     q, k, v = (rand_T((B, H, N, D), torch.float16, 60 + i) for i in range(3))
-    o = _lib.dense_attn_f16(q, k, _lib.v_tiles_f16(v), 1.0 / D ** 0.5, is_causal=causal)
+    o = _lib.dense_attn_f16(q, k, _lib.v_tiles_f16_swizzled(v), 1.0 / D ** 0.5, is_causal=causal)
     ref = torch.nn.functional.scaled_dot_product_attention(q.float(), k.float(), v.float(), is_causal=causal)
     met = oat.precision_metric(to_np(o), to_np(ref))
     assert met["Cossim"] > 0.9999 and met["L1"] < 5e-3, met
