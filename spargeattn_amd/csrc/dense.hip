@@ -11,6 +11,8 @@
 #include "launch.h"
 #include "lds_asm.h"
 
+#include <type_traits>
+
 namespace spg {
 
 typedef _Float16 v8h __attribute__((ext_vector_type(8)));
@@ -34,13 +36,15 @@ __device__ __forceinline__ uint32_t dense_k_swz(uint32_t row) {
   else return (row >> 1) & 7u;                       // two rows per line: bit 0 of the row is already a slot bit
 }
 
-template <int D>
-__global__ __launch_bounds__(256, 2) void dense_attn_f16_kernel(const DenseParams p) {
+template <int D, int NW>
+__global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void dense_attn_f16_kernel(const DenseParams p) {
   constexpr int KS = D / 16;          // k-steps of QK^T
   constexpr int NDT = D / 32;         // output channel tiles
   constexpr int TILE = 64 * D * 2;    // bytes of one K tile and of one V^T tile
   constexpr int CPR = D / 8;          // 16-byte chunks per K row
-  constexpr int WL = TILE / 4096;     // global_load_lds instructions per wavefront per tile
+  constexpr int QROWS = 32 * NW;      // query rows per workgroup
+  constexpr int BPQ = QROWS / 64;     // key blocks per query tile on the diagonal
+  constexpr int WL = TILE / (1024 * NW);   // global_load_lds instructions per wavefront per tile
   constexpr int NBUF = 2;
   __shared__ __align__(1024) unsigned char smem[NBUF * 2 * TILE];   // K ring | V^T ring
   const uint32_t lds_k0 = (uint32_t)(size_t)(__attribute__((address_space(3))) unsigned char *)smem;
@@ -54,8 +58,8 @@ __global__ __launch_bounds__(256, 2) void dense_attn_f16_kernel(const DenseParam
   const int tid = threadIdx.x, lane = tid & 63, r = lane & 31, hh = lane >> 5;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int N = p.N;
-  const int q_row = qb * 128 + wave * 32 + r;
-  const int nblk = p.is_causal ? min(p.nk, 2 * (qb + 1)) : p.nk;
+  const int q_row = qb * QROWS + wave * 32 + r;
+  const int nblk = p.is_causal ? min(p.nk, BPQ * (qb + 1)) : p.nk;
 
   v8h qreg[KS];
 #pragma unroll
@@ -129,11 +133,13 @@ __global__ __launch_bounds__(256, 2) void dense_attn_f16_kernel(const DenseParam
   __builtin_amdgcn_s_waitcnt(0x0F70);     // vmcnt(0)
   __syncthreads();
 
-#pragma unroll 1
-  for (int blk = 0; blk < nblk; blk++) {
-    const uint32_t so = (uint32_t)(blk & 1) * TILE;
-    // slot (blk+1)&1 was last read in iteration blk-1, which every wavefront has left (barrier at its end)
-    if (blk + 1 < nblk) load_tiles(blk + 1, (blk + 1) & 1);
+  // One key block.  SLOT = blk & 1 is a compile-time constant (the loop below is unrolled twice), so every LDS address
+  // of the step is a loop-invariant register plus an immediate offset.
+  auto step = [&](auto slot_tag, const int blk) __attribute__((always_inline)) {
+    constexpr int SLOT = decltype(slot_tag)::value;
+    constexpr int SO = SLOT * TILE;
+    // slot SLOT^1 was last read in iteration blk-1, which every wavefront has left (barrier at its end)
+    if (blk + 1 < nblk) load_tiles(blk + 1, SLOT ^ 1);
 
     // ---- S^T = K . Q^T: the reads of the second half of the k-steps are in flight while the first half multiplies
     v16f S0, S1;
@@ -143,11 +149,11 @@ __global__ __launch_bounds__(256, 2) void dense_attn_f16_kernel(const DenseParam
       constexpr int HK = KS / 2;
       v4i a0[KS], a1[KS];
 #pragma unroll
-      for (int ks = 0; ks < HK; ks++) lds_read_2x128<0, 16 * D * 2>(a0[ks], a1[ks], kaddr[ks] + so);
+      for (int ks = 0; ks < HK; ks++) lds_read_2x128<SO, SO + 16 * D * 2>(a0[ks], a1[ks], kaddr[ks]);
       if constexpr (HK == 4) { lds_wait4(a0[0], a1[0], a0[1], a1[1]); lds_wait4(a0[2], a1[2], a0[3], a1[3]); }
       else lds_wait4(a0[0], a1[0], a0[1], a1[1]);
 #pragma unroll
-      for (int ks = HK; ks < KS; ks++) lds_read_2x128<0, 16 * D * 2>(a0[ks], a1[ks], kaddr[ks] + so);
+      for (int ks = HK; ks < KS; ks++) lds_read_2x128<SO, SO + 16 * D * 2>(a0[ks], a1[ks], kaddr[ks]);
 #pragma unroll
       for (int ks = 0; ks < HK; ks++) {
         S0 = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(v8h, a0[ks]), qreg[ks], S0, 0, 0, 0);
@@ -163,7 +169,7 @@ __global__ __launch_bounds__(256, 2) void dense_attn_f16_kernel(const DenseParam
     }
 
     // slot e of this lane is key 64 blk + 32 hh + e (e < 16: S0[e], else S1[e - 16])
-    const bool edge = (p.is_causal && blk >= 2 * qb) || (blk == p.nk - 1);
+    const bool edge = (p.is_causal && blk >= BPQ * qb) || (blk == p.nk - 1);
     float x[32];
 #pragma unroll
     for (int e = 0; e < 32; e++) x[e] = e < 16 ? S0[e] : S1[e - 16];
@@ -209,19 +215,19 @@ __global__ __launch_bounds__(256, 2) void dense_attn_f16_kernel(const DenseParam
 
     // ---- O^T += V^T . P^T: key steps 0,1 are read first; steps 2,3 are in flight while 0,1 multiply
     {
-      const uint32_t va = va0 + so;
+      const uint32_t va = va0;
       v4i t[4][NDT];
 #pragma unroll
       for (int s4 = 0; s4 < 2; s4++) {
-        lds_read_2x128<0, 4096>(t[s4][0], t[s4][1], va ^ (uint32_t)(16 * s4));
-        if constexpr (NDT == 4) lds_read_2x128<8192, 12288>(t[s4][2], t[s4][3], va ^ (uint32_t)(16 * s4));
+        lds_read_2x128<SO, SO + 4096>(t[s4][0], t[s4][1], va ^ (uint32_t)(16 * s4));
+        if constexpr (NDT == 4) lds_read_2x128<SO + 8192, SO + 12288>(t[s4][2], t[s4][3], va ^ (uint32_t)(16 * s4));
       }
       if constexpr (NDT == 4) { lds_wait4(t[0][0], t[0][1], t[0][2], t[0][3]); lds_wait4(t[1][0], t[1][1], t[1][2], t[1][3]); }
       else { lds_wait4(t[0][0], t[0][1], t[1][0], t[1][1]); }
 #pragma unroll
       for (int s4 = 2; s4 < 4; s4++) {
-        lds_read_2x128<0, 4096>(t[s4][0], t[s4][1], va ^ (uint32_t)(16 * s4));
-        if constexpr (NDT == 4) lds_read_2x128<8192, 12288>(t[s4][2], t[s4][3], va ^ (uint32_t)(16 * s4));
+        lds_read_2x128<SO, SO + 4096>(t[s4][0], t[s4][1], va ^ (uint32_t)(16 * s4));
+        if constexpr (NDT == 4) lds_read_2x128<SO + 8192, SO + 12288>(t[s4][2], t[s4][3], va ^ (uint32_t)(16 * s4));
       }
 #pragma unroll
       for (int s4 = 0; s4 < 2; s4++)
@@ -238,6 +244,15 @@ __global__ __launch_bounds__(256, 2) void dense_attn_f16_kernel(const DenseParam
     }
     __builtin_amdgcn_s_waitcnt(0x0F70);   // this wavefront's share of block blk+1's tiles has landed in LDS
     __syncthreads();                      // block blk+1's tiles are complete; every wavefront is done with block blk's
+  };
+  {
+    int blk = 0;
+#pragma unroll 1
+    for (; blk + 2 <= nblk; blk += 2) {
+      step(std::integral_constant<int, 0>{}, blk);
+      step(std::integral_constant<int, 1>{}, blk + 1);
+    }
+    if (blk < nblk) step(std::integral_constant<int, 0>{}, blk);
   }
 
   const float dtot = half_swap_sum_f32(dsum);
@@ -262,13 +277,15 @@ hipError_t launch_dense_attn_f16(const void *q, const void *k, const void *vt, v
                                  float sm_scale, int is_causal, hipStream_t st) {
   DenseParams p;
   p.q = (const uint16_t *)q; p.k = (const uint16_t *)k; p.vt = (const uint16_t *)vt; p.out = (uint16_t *)out;
-  p.B = B; p.H = H; p.N = N; p.nq = (N + 127) / 128; p.nk = (N + 63) / 64;
+  // wavefronts (32 query rows each) per workgroup: 8 share a tile pair at D = 128 (one 64 KiB ring per CU), 4 at D = 64
+  const int NW = D == 64 ? 4 : 8;
+  p.B = B; p.H = H; p.N = N; p.nq = (N + 32 * NW - 1) / (32 * NW); p.nk = (N + 63) / 64;
   p.sm_scale_log2 = sm_scale * 1.44269504088896340736f;
   p.is_causal = is_causal;
   p.total_wg = p.nq * H * B;
   p.wg_per_xcd = (p.total_wg + 7) / 8;
-  if (D == 64) dense_attn_f16_kernel<64><<<p.wg_per_xcd * 8, 256, 0, st>>>(p);
-  else dense_attn_f16_kernel<128><<<p.wg_per_xcd * 8, 256, 0, st>>>(p);
+  if (D == 64) dense_attn_f16_kernel<64, 4><<<p.wg_per_xcd * 8, 256, 0, st>>>(p);
+  else dense_attn_f16_kernel<128, 8><<<p.wg_per_xcd * 8, 512, 0, st>>>(p);
   return hipGetLastError();
 }
 
