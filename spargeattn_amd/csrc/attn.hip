@@ -138,7 +138,11 @@ __global__ __launch_bounds__(256, PV16 ? 2 : 3) void block_sparse_attn_kernel(co
   constexpr int NBUF = 3;
   // LDS: K ring [NBUF][TILE] | V^T ring [NBUF][TILE] | votes
   __shared__ __align__(1024) unsigned char smem[NBUF * (TILE + VTILE)];
-  __shared__ int sVote[2][4];
+  // PV-skip vote of the per-block mode: a wavefront that votes "skip" stamps the iteration number into its slot; a slot
+  // that does not hold the current iteration number means "compute".  Only "skip" votes are written (they are rare at the
+  // thresholds in use), and only a wavefront that voted "skip" itself has to read the others' slots.  Two sets of slots,
+  // used alternately: a wavefront can be at most one barrier ahead of the slowest one.
+  __shared__ int sSkipAt[2][4];
   unsigned char *const sKr = smem;
   unsigned char *const sVr = smem + NBUF * TILE;
   const uint32_t lds_k0 = (uint32_t)(size_t)(__attribute__((address_space(3))) unsigned char *)smem;   // LDS byte address
@@ -280,6 +284,7 @@ __global__ __launch_bounds__(256, PV16 ? 2 : 3) void block_sparse_attn_kernel(co
   // 1/(2 pi) + dot * 2^-26, and the scores need no int-to-float conversion - the 2^26 goes into the multiplier and the
   // constant into the additive term of the fma that feeds exp2.
   const float acc_c = __builtin_bit_cast(float, (int)SPG_ACC_C_BITS);
+  if (tid < 8) (&sSkipAt[0][0])[tid] = -1;   // no slot may hold an iteration number by accident
   __builtin_amdgcn_s_waitcnt(0x0F70);     // vmcnt(0): Q fragment and the first tiles have arrived
   __syncthreads();
 
@@ -382,13 +387,13 @@ __global__ __launch_bounds__(256, PV16 ? 2 : 3) void block_sparse_attn_kernel(co
     fm = half_swap_max_raw(fm);
     const float diff = fm - m;
     const float m_new = max_raw(m, fm);
-    const float osc = __builtin_amdgcn_exp2f(m - m_new);
+    const float m_old = m;
     m = m_new;
     int vote = 1;
     if constexpr (!TAIL) {
       // max over rows of (diff) + thr > 0  <=>  some row has diff + thr > 0 (fp32 addition is monotonic)
       vote = __any(diff + thr > 0.f);
-      if (lane == 0) sVote[it & 1][wave] = vote;
+      if (vote == 0 && lane == 0) sSkipAt[it & 1][wave] = it;
     }
     __builtin_amdgcn_s_waitcnt(0x0F70);   // this wave's share of block it+1's tiles has landed in LDS
     __syncthreads();   // block it+1's tiles are complete; the votes are visible; ring slot of block it-1 is free
@@ -398,7 +403,8 @@ __global__ __launch_bounds__(256, PV16 ? 2 : 3) void block_sparse_attn_kernel(co
       // per-block mode: a wavefront whose own vote is set knows the OR already; only one that voted "skip" has to read
       // what the others wrote (an LDS round trip that the common case does without)
       if (p.pv_mode == 1 && !compute)
-        compute = (sVote[it & 1][0] | sVote[it & 1][1] | sVote[it & 1][2] | sVote[it & 1][3]) != 0;
+        compute = !(sSkipAt[it & 1][0] == it && sSkipAt[it & 1][1] == it && sSkipAt[it & 1][2] == it &&
+                    sSkipAt[it & 1][3] == it);
     }
     if (!TAIL || it + 2 < nv) {
       if constexpr (CS) {
@@ -408,8 +414,11 @@ __global__ __launch_bounds__(256, PV16 ? 2 : 3) void block_sparse_attn_kernel(co
         SPG_LOAD_TILES(blk2, b2);
       }
     }
-    dsum *= osc;
-    if (__any(osc != 1.0f)) {
+    // the running maximum of some query rose: rescale (exp2(0) = 1 exactly, so the other iterations need neither the
+    // exponential nor the products)
+    if (__any(diff > 0.f)) {
+      const float osc = __builtin_amdgcn_exp2f(m_old - m_new);
+      dsum *= osc;
 #pragma unroll
       for (int dt = 0; dt < NDT; dt++)
 #pragma unroll
@@ -418,7 +427,7 @@ __global__ __launch_bounds__(256, PV16 ? 2 : 3) void block_sparse_attn_kernel(co
     if (compute) {
       cnt++;
       const float neg0 = PV16 ? -m : -m + SPG_FP8_OFFSET;
-      float ps = 0.f;
+      float ps;
       float x[32];
       if constexpr (!TAIL) {
         // three passes kept apart for the scheduler: a multiply-add feeding the exponential of the same element directly,
@@ -440,10 +449,12 @@ __global__ __launch_bounds__(256, PV16 ? 2 : 3) void block_sparse_attn_kernel(co
         for (int e = 0; e < 32; e++) x[e] = __builtin_amdgcn_exp2f(x[e]);
         __builtin_amdgcn_sched_barrier(0);
         if constexpr (!PV16) {
+          ps = x[0];
 #pragma unroll
-          for (int e = 0; e < 32; e++) ps += x[e];
+          for (int e = 1; e < 32; e++) ps += x[e];
         }
       } else {
+        ps = 0.f;
         const float masked = __builtin_fmaf(SPG_NEG_BIG, c, neg0);   // what the sentinel score turns into
         const float dq26 = dq * SPG_ACC_SCALE;
 #pragma unroll
