@@ -167,6 +167,36 @@ def test_similarity_flag_on_degenerate_rows(dtype, thr_value):
         assert np.array_equal(ref_sim_128(x, thr, tag), want)
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("thr_value", [-0.1, 0.2])
+@pytest.mark.parametrize("N", [64 * 7 + 13, 64 * 6 + 5, 64 * 5, 64 * 4 + 64, 50])
+@pytest.mark.parametrize("D", [64, 128])
+def test_pool_sim_quant_two_blocks_per_workgroup(dtype, thr_value, N, D):
+    """A workgroup covers 128 rows, i.e. two 64-row blocks: the second one may be partial, full, or absent, and a
+    degenerate row (all zero, infinity) in one block must not change the other block's flag, scale or pooled mean."""
+    B, H = 1, 2
+    tag = tag_of(dtype)
+    k = rand_T((B, H, N, D), dtype, 21, shift=0.25)
+    if N > 70:
+        k[0, 0, 3] = 0                             # block 0 of head 0: an all-zero row before centring
+        k[0, 1, 64 + 2, 5] = float("inf")          # block 1 of head 1
+    thr = torch.tensor([thr_value] * H, dtype=torch.float32, device="cuda")
+    km = _lib.km_mean(k)
+    for mean in (km, None):
+        pool, sim, xq, scale = _lib.pool_sim_quant(k, mean, 64, thr)
+        ref = mp.pool_sim_quant(to_np(k), None if mean is None else to_np(mean[:, :, 0]), 64, thr.cpu().numpy(), tag)
+        assert np.array_equal(sim.cpu().numpy(), ref["sim"]), (sim.cpu().numpy(), ref["sim"])
+        finite = np.isfinite(ref["scale"])        # an infinity in a block makes its scale and codes undefined
+        assert np.array_equal(scale.cpu().numpy()[finite].view(np.uint32), ref["scale"][finite].view(np.uint32))
+        nb = ref["scale"].shape[-1]
+        rows_ok = np.repeat(finite, 64, axis=-1)[..., :N]
+        assert np.array_equal(xq.cpu().numpy()[rows_ok], ref["q"][rows_ok])
+        got_pool, want_pool = to_np(pool), ref["pool"]
+        ok = np.isfinite(want_pool)
+        assert np.array_equal(got_pool[ok], want_pool[ok])
+        assert nb == (N + 63) // 64
+
+
 def ref_sim_128(x, thr, tag):
     return mp.pool_sim_quant(to_np(x), None, 128, thr.cpu().numpy(), tag)["sim"]
 
