@@ -496,6 +496,23 @@ __device__ __forceinline__ void emit_lut(FlagFn flag, int nk, int nkp, int32_t *
   if (tid == 0) *valid_out = st.y;
 }
 
+// binary64 -> 16-bit pattern (round to nearest even) through binary32 where that provably gives the same bits: the
+// first rounding (to 24 bits) can only change the second one when it lands exactly on a rounding tie of the 16-bit
+// format, so every other value inside the format's normal range takes two hardware conversions instead of the 64-bit
+// integer arithmetic of f64_to_elem; ties, zero-range, subnormal and overflowing values go the exact way.
+template <int DT>
+__device__ __forceinline__ uint16_t f64_to_elem_fast(double x) {
+  const float r = (float)x;                                        // v_cvt_f32_f64
+  const uint32_t b = __builtin_bit_cast(uint32_t, r);
+  const uint32_t mag = b & 0x7fffffffu;
+  constexpr uint32_t DROP = DT == 1 ? 16u : 13u;                   // binary32 mantissa bits the 16-bit format drops
+  constexpr uint32_t LOW = (1u << DROP) - 1u, TIE = 1u << (DROP - 1u);
+  constexpr uint32_t LO = DT == 1 ? 0x00800000u : 0x38800000u;     // 2^-126 / 2^-14: smallest normal of the format
+  constexpr uint32_t HI = DT == 1 ? 0x7f000000u : 0x47000000u;     // 2^127 / 2^15: well below the overflow threshold
+  const bool safe = mag == 0u || (mag >= LO && mag < HI && (b & LOW) != TIE);
+  return safe ? f32_to_elem<DT>(r) : f64_to_elem<DT>(x);
+}
+
 // =============================================================================================
 // block_select: one workgroup per (R consecutive q block rows, b*h).
 // Phase 1 computes the R x nk pooled scores with every pooled-K row read ONCE for the R rows (one lane per
@@ -676,11 +693,12 @@ __global__ __launch_bounds__(256) void block_select_kernel(
 
 // =============================================================================================
 // block_select, wavefront-per-row variant (nk <= 2048).
-// Phase 1 is the same score computation, two columns per lane at a time so that one broadcast LDS read of pooled Q
-// feeds four multiply-adds.  Phase 2 gives each of the four wavefronts its own rows and keeps a whole row in
-// registers (EPL = nkp / 64 columns per lane): no workgroup barrier, the stable descending sort is a bitonic network
+// Phase 1 computes the scores of 16 pooled-Q rows against all pooled-K rows on the matrix unit in binary64
+// (v_mfma_f64_16x16x4_f64: operands are delivered once per 1024 multiply-adds instead of once per multiply-add) and
+// leaves them in LDS as 16-bit patterns.  Phase 2 gives each of the four wavefronts its own rows and keeps a whole row
+// in registers (EPL = nkp / 64 columns per lane): no workgroup barrier, the stable descending sort is a bitonic network
 // whose short-distance steps are register-local and whose long-distance steps are lane exchanges.
-// dynamic LDS: R*D*8 (pooled Q as doubles) + R*nkp*4 (scores) + 4*nkp*4 (per-wave index list) + 4*64*8 (lane sums).
+// dynamic LDS: 16*nkp*2 (scores) + 4*nkp*4 (per-wave index list) + 4*64*8 (lane sums).
 // =============================================================================================
 template <int EPL, int K, int J>
 __device__ __forceinline__ void bitonic_step(uint32_t (&key)[EPL], int lane) {
@@ -727,18 +745,19 @@ __device__ __forceinline__ void bitonic_sort_desc(uint32_t (&key)[EPL], int lane
   if constexpr (K < 64 * EPL) bitonic_sort_desc<EPL, K * 2>(key, lane);
 }
 
-template <int D, int DT, int R, int EPL>
-__global__ __launch_bounds__(256) void block_select_wave_kernel(
+template <int D, int DT, int NW, int EPL>
+__global__ __launch_bounds__(64 * NW) void block_select_wave_kernel(
     const uint16_t *__restrict__ pool_q, const uint8_t *__restrict__ sim_q, const uint16_t *__restrict__ pool_k,
     const uint8_t *__restrict__ sim_k, const float *__restrict__ topk, const float *__restrict__ cdfthr, int is_causal,
     int sink, int32_t *__restrict__ lut, int32_t *__restrict__ valid, uint8_t *__restrict__ bmap, int H, int Hkv, int nq,
     int nk) {
+  constexpr int R = 16;             // rows per workgroup: phase 1 computes 16 x 16 score tiles on the matrix unit
   constexpr int NKP = 64 * EPL;
+  static_assert(NW == 8 || NW == 16, "wavefronts per workgroup");
   extern __shared__ __align__(16) unsigned char smem[];
-  double *s_pq = (double *)smem;                                              // [R][D]
-  float *s_scores = (float *)(smem + (size_t)R * D * 8);                      // [R][NKP]
-  int32_t *s_idx_all = (int32_t *)(smem + (size_t)R * D * 8 + (size_t)R * NKP * 4);   // [4][NKP]
-  double *s_lsum_all = (double *)(smem + (size_t)R * D * 8 + (size_t)R * NKP * 4 + 4 * (size_t)NKP * 4);   // [4][64]
+  uint16_t *s_scores = (uint16_t *)smem;                                      // [R][NKP] scores as 16-bit patterns
+  uint16_t *s_idx_all = (uint16_t *)(smem + (size_t)R * NKP * 2);             // [NW][NKP] (column indices are below 2048)
+  double *s_lsum_all = (double *)(smem + (size_t)R * NKP * 2 + NW * (size_t)NKP * 2);   // [NW][64]
 
   // Causal rows get heavier with the row index.  Workgroups that differ by 8 in blockIdx.y tend to share a CU (ids are
   // dealt round-robin over 8 XCDs, then over the CUs of an XCD), so the row-group index is rotated by a quarter of
@@ -746,11 +765,8 @@ __global__ __launch_bounds__(256) void block_select_wave_kernel(
   const int bx = (int)((blockIdx.x + (blockIdx.y >> 3) * (gridDim.x >> 2)) % gridDim.x);
   const int i0 = bx * R, bh = blockIdx.y, h = bh % H, tid = threadIdx.x;
   const int rows = min(R, nq - i0);
-  for (int t = tid; t < R * D; t += 256) {
-    const int row = t / D;
-    s_pq[t] = row < rows ? (double)elem_to_f32<DT>(pool_q[((size_t)bh * nq + i0 + row) * D + (t % D)]) : 0.0;
-  }
-  __syncthreads();
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
 
   const float sm_scale = (D == 64) ? 0.125f : 0.088388347648318447f;  // fp32(D^-0.5)
   // grouped K/V heads: query head h is scored against the pooled blocks of K head h / (H / Hkv)
@@ -758,89 +774,112 @@ __global__ __launch_bounds__(256) void block_select_wave_kernel(
   const uint16_t *pk_base = pool_k + (size_t)bhk * nk * D;
   const uint8_t *simk = sim_k + (size_t)bhk * nk;
 
-  // ---- phase 1: scores, binary64 accumulation in the fixed order d = 0..D-1 (products of 16-bit floats are exact) ----
-  // columns at or beyond j_live are masked for every row of this workgroup: no arithmetic for them
-  const int j_live = is_causal ? min(nk, 2 * (i0 + rows)) : nk;
-  for (int jb = 0; jb < NKP; jb += 512) {
-    const int ja = jb + tid, jc = jb + 256 + tid;
-    const bool live_a = ja < j_live, live_c = jc < j_live;
-    double acc_a[R], acc_c[R];
+  // ---- phase 1: the 16 x nk pooled scores in binary64 on the matrix unit (v_mfma_f64_16x16x4_f64) --------------------
+  // Products of two 16-bit floats are exact in binary64 and so are their partial sums (the contract's domain), so the
+  // sum does not depend on the order of the terms: a tile of 16 rows x 16 columns accumulates the D dimensions four at a
+  // time.  Lane l = 16 g + c supplies A[c][g] (pooled Q row c) and B[g][c] (pooled K column c) of each step and receives
+  // rows g, g + 4, g + 8, g + 12 of column c.  Step s pairs lane group g with dimension 32 (s / 8) + 8 g + (s % 8): every lane
+  // then consumes the eight values of one 16-byte load in eight consecutive steps.
+  {
+    typedef double d4_t __attribute__((ext_vector_type(4)));
+    constexpr int NL = D / 32;                    // 16-byte loads per row and lane
+    const int c = lane & 15, g = lane >> 4;
+    double qa[D / 4];
+    {
+      const bool row_ok = c < rows;
+      const uint16_t *qrow = pool_q + ((size_t)bh * nq + i0 + (row_ok ? c : 0)) * D + 8 * g;
 #pragma unroll
-    for (int row = 0; row < R; row++) { acc_a[row] = 0.0; acc_c[row] = 0.0; }
-    if (jb < j_live) {                                               // workgroup-uniform
-      const uint4 *krow_a = (const uint4 *)(pk_base + (size_t)(live_a ? ja : 0) * D);
-      const uint4 *krow_c = (const uint4 *)(pk_base + (size_t)(live_c ? jc : 0) * D);
-      const bool two = jb + 256 < j_live;                            // workgroup-uniform
-      uint4 va_next = krow_a[0], vc_next = krow_c[0];
-#pragma unroll 1
-      for (int cch = 0; cch < D / 8; cch++) {
-        const uint4 va = va_next, vc_cur = vc_next;
-        const int nxt = min(cch + 1, D / 8 - 1);                     // the next chunk is in flight during this one
-        va_next = krow_a[nxt];
-        vc_next = krow_c[nxt];
-        const uint32_t wa[4] = {va.x, va.y, va.z, va.w};
-        double ka[8];
+      for (int t = 0; t < NL; t++) {
+        const uint4 v = row_ok ? *(const uint4 *)(qrow + 32 * t) : make_uint4(0, 0, 0, 0);
+        const uint32_t w[4] = {v.x, v.y, v.z, v.w};
 #pragma unroll
         for (int e = 0; e < 8; e++)
-          ka[e] = (double)elem_to_f32<DT>((uint16_t)((e & 1) ? (wa[e >> 1] >> 16) : (wa[e >> 1] & 0xffffu)));
-        if (two) {
-          const uint32_t wc[4] = {vc_cur.x, vc_cur.y, vc_cur.z, vc_cur.w};
-          double kc[8];
+          qa[8 * t + e] = (double)elem_to_f32<DT>((uint16_t)((e & 1) ? (w[e >> 1] >> 16) : (w[e >> 1] & 0xffffu)));
+      }
+    }
+    // columns at or beyond j_live are masked for every row of this workgroup: they get -inf without any arithmetic
+    const int j_live = is_causal ? min(nk, 2 * (i0 + rows)) : nk;
+    constexpr uint16_t NEG_INF = DT == 1 ? 0xff80u : 0xfc00u;
+    const int n_tiles = NKP / 16, live_tiles = (j_live + 15) / 16;
+    auto load_k = [&](int ct, uint4 (&raw)[NL]) __attribute__((always_inline)) {
+      const int j = min(16 * ct + c, nk - 1);    // columns beyond nk re-read the last one and are masked below
+      const uint16_t *krow = pk_base + (size_t)j * D + 8 * g;
 #pragma unroll
-          for (int e = 0; e < 8; e++)
-            kc[e] = (double)elem_to_f32<DT>((uint16_t)((e & 1) ? (wc[e >> 1] >> 16) : (wc[e >> 1] & 0xffffu)));
+      for (int t = 0; t < NL; t++) raw[t] = *(const uint4 *)(krow + 32 * t);
+    };
+    auto finish = [&](int ct, const d4_t &acc) __attribute__((always_inline)) {
+      const int j = 16 * ct + c;
+      const bool dead = j >= nk || simk[min(j, nk - 1)] == 0;
 #pragma unroll
-          for (int row = 0; row < R; row++) {
-            const double *q = s_pq + row * D + cch * 8;
+      for (int v = 0; v < 4; v++) {
+        const int row = g + 4 * v;
+        const float a1 = elem_to_f32<DT>(f64_to_elem_fast<DT>(acc[v]));
+        uint16_t a2 = f64_to_elem_fast<DT>((double)a1 * (double)sm_scale);
+        if (dead || (is_causal && j >= 2 * (i0 + row + 1))) a2 = NEG_INF;
+        s_scores[(size_t)row * NKP + j] = a2;
+      }
+    };
+    // NW = 8: two column tiles per trip (two independent accumulator chains); NW = 16: one (the register budget of a
+    // 1024-thread workgroup is 128 per lane; four wavefronts per SIMD keep the matrix unit busy instead).  The next
+    // trip's pooled-K rows are in flight meanwhile.
+    constexpr bool DUAL = NW == 8;
+    constexpr int STEP = DUAL ? 2 * NW : NW;
+    uint4 ra[NL], rb[DUAL ? NL : 1];
+    int ct = wave;
+    if (ct < live_tiles) {
+      load_k(ct, ra);
+      if constexpr (DUAL) load_k(min(ct + NW, live_tiles - 1), rb);
+    }
+#pragma unroll 1
+    for (; ct < live_tiles; ct += STEP) {
+      uint4 ka[NL], kb[DUAL ? NL : 1];
 #pragma unroll
-            for (int e = 0; e < 8; e++) {
-              const double qe = q[e];
-              acc_a[row] = __builtin_fma(qe, ka[e], acc_a[row]);
-              acc_c[row] = __builtin_fma(qe, kc[e], acc_c[row]);
-            }
-          }
-        } else {
+      for (int t = 0; t < NL; t++) { ka[t] = ra[t]; if constexpr (DUAL) kb[t] = rb[t]; }
+      const bool two = DUAL && ct + NW < live_tiles;         // wavefront-uniform
+      if (ct + STEP < live_tiles) {
+        load_k(ct + STEP, ra);
+        if constexpr (DUAL) load_k(min(ct + STEP + NW, live_tiles - 1), rb);
+      }
+      d4_t acc_a = {0.0, 0.0, 0.0, 0.0}, acc_b = {0.0, 0.0, 0.0, 0.0};
 #pragma unroll
-          for (int row = 0; row < R; row++) {
-            const double *q = s_pq + row * D + cch * 8;
+      for (int t = 0; t < NL; t++) {
+        const uint32_t wa[4] = {ka[t].x, ka[t].y, ka[t].z, ka[t].w};
 #pragma unroll
-            for (int e = 0; e < 8; e++) acc_a[row] = __builtin_fma(q[e], ka[e], acc_a[row]);
+        for (int e = 0; e < 8; e++) {
+          const double xa = (double)elem_to_f32<DT>((uint16_t)((e & 1) ? (wa[e >> 1] >> 16) : (wa[e >> 1] & 0xffffu)));
+          acc_a = __builtin_amdgcn_mfma_f64_16x16x4f64(qa[8 * t + e], xa, acc_a, 0, 0, 0);
+          if constexpr (DUAL) {
+            const uint32_t wb[4] = {kb[t].x, kb[t].y, kb[t].z, kb[t].w};
+            const double xb = (double)elem_to_f32<DT>((uint16_t)((e & 1) ? (wb[e >> 1] >> 16) : (wb[e >> 1] & 0xffffu)));
+            acc_b = __builtin_amdgcn_mfma_f64_16x16x4f64(qa[8 * t + e], xb, acc_b, 0, 0, 0);
           }
         }
       }
+      finish(ct, acc_a);
+      if (two) finish(ct + NW, acc_b);
     }
-    const bool dead_a = !live_a || simk[ja] == 0, dead_c = !live_c || simk[jc] == 0;
+    // dead column tiles
+    for (int t2 = live_tiles + wave; t2 < n_tiles; t2 += NW) {
+      const int j = 16 * t2 + c;
 #pragma unroll
-    for (int row = 0; row < R; row++) {
-      const float a1 = elem_to_f32<DT>(f64_to_elem<DT>(acc_a[row]));
-      float a2 = elem_to_f32<DT>(f64_to_elem<DT>((double)a1 * (double)sm_scale));
-      if (dead_a || (is_causal && ja >= 2 * (i0 + row + 1))) a2 = -INFINITY;
-      s_scores[(size_t)row * NKP + ja] = a2;
-      if (NKP > 256) {
-        const float c1 = elem_to_f32<DT>(f64_to_elem<DT>(acc_c[row]));
-        float c2 = elem_to_f32<DT>(f64_to_elem<DT>((double)c1 * (double)sm_scale));
-        if (dead_c || (is_causal && jc >= 2 * (i0 + row + 1))) c2 = -INFINITY;
-        s_scores[(size_t)row * NKP + jc] = c2;
-      }
+      for (int v = 0; v < 4; v++) s_scores[(size_t)(g + 4 * v) * NKP + j] = NEG_INF;
     }
   }
   __syncthreads();
 
-  // ---- phase 2: wavefront `wave` owns rows wave, wave + 4, ...; lane l holds columns l, l + 64, ... ----------------
-  const int lane = tid & 63;
-  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  int32_t *s_idx = s_idx_all + wave * NKP;
+  // ---- phase 2: wavefront `wave` owns rows wave, wave + NW, ...; lane l holds columns l, l + 64, ... ---------------
+  uint16_t *s_idx = s_idx_all + wave * NKP;
   double *s_lsum = s_lsum_all + wave * 64;
-  for (int row = wave; row < rows; row += 4) {
+  for (int row = wave; row < rows; row += NW) {
     const int i = i0 + row;
     const int causal_lim = is_causal ? min(nk, 2 * (i + 1)) : nk;
-    const float *s_score = s_scores + (size_t)row * NKP;
+    const uint16_t *s_score = s_scores + (size_t)row * NKP;
 
     float sc[EPL];
     float lmax = -INFINITY;
 #pragma unroll
     for (int t = 0; t < EPL; t++) {
-      sc[t] = s_score[t * 64 + lane];               // columns >= nk were written as -inf by phase 1
+      sc[t] = elem_to_f32<DT>(s_score[t * 64 + lane]);   // columns >= nk were written as -inf by phase 1
       lmax = fmaxf(lmax, sc[t]);
     }
     const float mx = wave_max_f32(lmax);
@@ -857,14 +896,28 @@ __global__ __launch_bounds__(256) void block_select_wave_kernel(
     for (int o = 32; o >= 1; o >>= 1) part = part + shfl_xor_f64(part, o);
     const double total = part;
 
-    // probabilities -> sortable keys (value bits, then lower column first)
+    // probabilities -> sortable keys (value bits, then lower column first).  The 16-bit pattern of e / total is taken
+    // from e * (1 / total), which is within two units in the last place of the quotient: through binary32, the two
+    // agree unless the product lands exactly on a rounding tie of the 16-bit format or outside its normal range, and
+    // those elements take the division and the exact conversion.
+    const double rtotal = total > 0.0 ? 1.0 / total : 0.0;     // a row without a live column has e = 0 everywhere
     uint32_t okey[EPL], key[EPL];
 #pragma unroll
     for (int t = 0; t < EPL; t++) {
       const int j = t * 64 + lane;
-      double p = ev[t] / total;
-      if (!__builtin_isfinite(p)) p = 0.0;
-      const uint32_t bits = f64_to_elem<DT>(p);
+      const float pr = (float)(ev[t] * rtotal);
+      const uint32_t pb = __builtin_bit_cast(uint32_t, pr);    // probabilities are non-negative
+      constexpr uint32_t DROP = DT == 1 ? 16u : 13u, LOWM = (1u << DROP) - 1u, TIE = 1u << (DROP - 1u);
+      constexpr uint32_t LO = DT == 1 ? 0x00800000u : 0x38800000u;     // smallest normal of the format
+      const bool safe = pb == 0u || (pb >= LO && pb <= 0x3f800000u && (pb & LOWM) != TIE);
+      uint32_t bits;
+      if (safe) {
+        bits = f32_to_elem<DT>(pr);
+      } else {
+        double p = ev[t] / total;
+        if (!__builtin_isfinite(p)) p = 0.0;
+        bits = f64_to_elem<DT>(p);
+      }
       okey[t] = j < nk ? ((bits << 16) | (0xffffu - (uint32_t)j)) : 0u;
       key[t] = okey[t];
     }
@@ -947,7 +1000,7 @@ __global__ __launch_bounds__(256) void block_select_wave_kernel(
       }
       const unsigned long long m = __ballot(f);
       const int below = __builtin_amdgcn_mbcnt_hi((uint32_t)(m >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)m, 0));
-      if (f) s_idx[base + below] = j;
+      if (f) s_idx[base + below] = (uint16_t)j;
       base += __builtin_popcountll(m);
     }
     __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
@@ -957,7 +1010,7 @@ __global__ __launch_bounds__(256) void block_select_wave_kernel(
       const int pidx = t * 64 + lane;
       if (pidx < nk) {
         int v = 0;
-        if (pidx < base) v = s_idx[pidx] - (pidx ? s_idx[pidx - 1] : 0);
+        if (pidx < base) v = (int)s_idx[pidx] - (pidx ? (int)s_idx[pidx - 1] : 0);
         lut[row_off + pidx] = v;
       }
     }
@@ -1134,22 +1187,24 @@ static hipError_t launch_bs2(const void *pq, const uint8_t *sq, const void *pk, 
   const int nkp = next_pow2_ge(nk, 256);
   if (nkp <= 2048) {
     // a whole row fits the registers of one wavefront
-#define SPG_BSW(R_, EPL_)                                                                                       \
+#define SPG_BSW(NW_, EPL_)                                                                                      \
     {                                                                                                           \
-      const size_t lds = (size_t)R_ * D * 8 + (size_t)R_ * nkp * 4 + 16 * (size_t)nkp + 4 * 64 * 8;             \
-      auto kern = block_select_wave_kernel<D, DT, R_, EPL_>;                                                    \
+      const size_t lds = (size_t)16 * nkp * 2 + (size_t)NW_ * nkp * 2 + NW_ * 64 * 8;                           \
+      auto kern = block_select_wave_kernel<D, DT, NW_, EPL_>;                                                   \
       {                                                                                                         \
-        hipError_t e = allow_dynamic_lds<block_select_wave_kernel<D, DT, R_, EPL_>>(lds);                       \
+        hipError_t e = allow_dynamic_lds<block_select_wave_kernel<D, DT, NW_, EPL_>>(lds);                      \
         if (e != hipSuccess) return e;                                                                          \
       }                                                                                                         \
-      kern<<<dim3((nq + R_ - 1) / R_, B * H), 256, lds, st>>>((const uint16_t *)pq, sq, (const uint16_t *)pk, sk, topk, \
-                                                              cdf, causal, sink, lut, valid, bmap, H, Hkv, nq, nk); \
+      kern<<<dim3((nq + 15) / 16, B * H), 64 * NW_, lds, st>>>((const uint16_t *)pq, sq, (const uint16_t *)pk, sk, topk, \
+                                                               cdf, causal, sink, lut, valid, bmap, H, Hkv, nq, nk); \
       return hipSuccess;                                                                                        \
     }
-    if (nkp == 256) SPG_BSW(8, 4)
-    if (nkp == 512) SPG_BSW(8, 8)
-    if (nkp == 1024) SPG_BSW(8, 16)
-    SPG_BSW(4, 32)
+    // one wavefront per row (16 per workgroup) where a row's registers fit the 128 a 1024-thread workgroup leaves each
+    // lane, two rows per wavefront beyond
+    if (nkp == 256) SPG_BSW(16, 4)
+    if (nkp == 512) SPG_BSW(16, 8)
+    if (nkp == 1024) SPG_BSW(16, 16)
+    SPG_BSW(8, 32)
 #undef SPG_BSW
   }
   // rows per workgroup: reuse of the pooled-K reads against LDS footprint (scores are R*nkp floats)
