@@ -745,8 +745,8 @@ __device__ __forceinline__ void bitonic_sort_desc(uint32_t (&key)[EPL], int lane
   if constexpr (K < 64 * EPL) bitonic_sort_desc<EPL, K * 2>(key, lane);
 }
 
-template <int D, int DT, int NW, int EPL>
-__global__ __launch_bounds__(64 * NW) void block_select_wave_kernel(
+template <int D, int DT, int NW, int EPL, bool DUAL>
+__global__ __launch_bounds__(64 * NW, (!DUAL && NW == 8) ? 2 : 1) void block_select_wave_kernel(
     const uint16_t *__restrict__ pool_q, const uint8_t *__restrict__ sim_q, const uint16_t *__restrict__ pool_k,
     const uint8_t *__restrict__ sim_k, const float *__restrict__ topk, const float *__restrict__ cdfthr, int is_causal,
     int sink, int32_t *__restrict__ lut, int32_t *__restrict__ valid, uint8_t *__restrict__ bmap, int H, int Hkv, int nq,
@@ -819,10 +819,9 @@ __global__ __launch_bounds__(64 * NW) void block_select_wave_kernel(
         s_scores[(size_t)row * NKP + j] = a2;
       }
     };
-    // NW = 8: two column tiles per trip (two independent accumulator chains); NW = 16: one (the register budget of a
-    // 1024-thread workgroup is 128 per lane; four wavefronts per SIMD keep the matrix unit busy instead).  The next
-    // trip's pooled-K rows are in flight meanwhile.
-    constexpr bool DUAL = NW == 8;
+    // DUAL: two column tiles per trip (two independent accumulator chains), for the long rows that leave a SIMD only two
+    // wavefronts; otherwise one (128 registers per lane, four wavefronts per SIMD keep the matrix unit busy instead).
+    // The next trip's pooled-K rows are in flight meanwhile.
     constexpr int STEP = DUAL ? 2 * NW : NW;
     uint4 ra[NL], rb[DUAL ? NL : 1];
     int ct = wave;
@@ -1187,12 +1186,12 @@ static hipError_t launch_bs2(const void *pq, const uint8_t *sq, const void *pk, 
   const int nkp = next_pow2_ge(nk, 256);
   if (nkp <= 2048) {
     // a whole row fits the registers of one wavefront
-#define SPG_BSW(NW_, EPL_)                                                                                      \
+#define SPG_BSW(NW_, EPL_, DUAL_)                                                                                    \
     {                                                                                                           \
       const size_t lds = (size_t)16 * nkp * 2 + (size_t)NW_ * nkp * 2 + NW_ * 64 * 8;                           \
-      auto kern = block_select_wave_kernel<D, DT, NW_, EPL_>;                                                   \
+      auto kern = block_select_wave_kernel<D, DT, NW_, EPL_, DUAL_>;                                                   \
       {                                                                                                         \
-        hipError_t e = allow_dynamic_lds<block_select_wave_kernel<D, DT, NW_, EPL_>>(lds);                      \
+        hipError_t e = allow_dynamic_lds<block_select_wave_kernel<D, DT, NW_, EPL_, DUAL_>>(lds);                      \
         if (e != hipSuccess) return e;                                                                          \
       }                                                                                                         \
       kern<<<dim3((nq + 15) / 16, B * H), 64 * NW_, lds, st>>>((const uint16_t *)pq, sq, (const uint16_t *)pk, sk, topk, \
@@ -1201,10 +1200,10 @@ static hipError_t launch_bs2(const void *pq, const uint8_t *sq, const void *pk, 
     }
     // one wavefront per row (16 per workgroup) where a row's registers fit the 128 a 1024-thread workgroup leaves each
     // lane, two rows per wavefront beyond
-    if (nkp == 256) SPG_BSW(16, 4)
-    if (nkp == 512) SPG_BSW(16, 8)
-    if (nkp == 1024) SPG_BSW(16, 16)
-    SPG_BSW(8, 32)
+    if (nkp == 256) SPG_BSW(8, 4, false)
+    if (nkp == 512) SPG_BSW(8, 8, false)
+    if (nkp == 1024) SPG_BSW(8, 16, false)
+    SPG_BSW(8, 32, true)
 #undef SPG_BSW
   }
   // rows per workgroup: reuse of the pooled-K reads against LDS footprint (scores are R*nkp floats)
