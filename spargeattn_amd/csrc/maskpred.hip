@@ -59,13 +59,23 @@ __global__ __launch_bounds__(256) void km_partial_kernel(const uint16_t *__restr
   }
 }
 
+// One workgroup per (batch, head), blockDim = (D, 8): eight threads share a column's partial sums (exact, so the order of
+// the additions is free), thread (d, 0) adds the eight sub-sums and rounds.
 template <int DT>
 __global__ void km_final_kernel(const double *__restrict__ part, uint16_t *__restrict__ km, int nchunk, int D, int N) {
-  const int bh = blockIdx.x, d = threadIdx.x;
+  __shared__ double s_sub[8][128];
+  const int bh = blockIdx.x, d = threadIdx.x, y = threadIdx.y;
   double s = 0.0;
-#pragma unroll 16
-  for (int i = 0; i < nchunk; i++) s += part[((size_t)bh * nchunk + i) * D + d];
-  km[(size_t)bh * D + d] = f64_to_elem<DT>(s / (double)N);
+#pragma unroll 4
+  for (int i = y; i < nchunk; i += 8) s += part[((size_t)bh * nchunk + i) * D + d];
+  s_sub[y][d] = s;
+  __syncthreads();
+  if (y == 0) {
+    double t = 0.0;
+#pragma unroll
+    for (int u = 0; u < 8; u++) t += s_sub[u][d];
+    km[(size_t)bh * D + d] = f64_to_elem<DT>(t / (double)N);
+  }
 }
 
 // =============================================================================================
@@ -1074,7 +1084,7 @@ static void launch_km(const void *k, Strides ks, void *km, void *ws, int B, int 
   const int nchunk = km_chunks(B, H, N);
   const int rpc = (N + nchunk - 1) / nchunk;
   km_partial_kernel<D, DT><<<dim3(nchunk, B * H), 256, 0, st>>>((const uint16_t *)k, ks, H, (double *)ws, N, rpc);
-  km_final_kernel<DT><<<B * H, D, 0, st>>>((const double *)ws, (uint16_t *)km, nchunk, D, N);
+  km_final_kernel<DT><<<B * H, dim3(D, 8), 0, st>>>((const double *)ws, (uint16_t *)km, nchunk, D, N);
 }
 
 void launch_km_mean(const void *k, Strides ks, void *km, void *ws, int B, int H, int N, int D, int dtype, hipStream_t st) {
