@@ -124,6 +124,23 @@ __global__ __launch_bounds__(256) void div_selftest_kernel(unsigned long long *c
   atomicAdd(&counts[1], bad);
 }
 
+// binary64 -> 16-bit pattern (round to nearest even) through binary32 where that provably gives the same bits: the
+// first rounding (to 24 bits) can only change the second one when it lands exactly on a rounding tie of the 16-bit
+// format, so every other value inside the format's normal range takes two hardware conversions instead of the 64-bit
+// integer arithmetic of f64_to_elem; ties, zero-range, subnormal and overflowing values go the exact way.
+template <int DT>
+__device__ __forceinline__ uint16_t f64_to_elem_fast(double x) {
+  const float r = (float)x;                                        // v_cvt_f32_f64
+  const uint32_t b = __builtin_bit_cast(uint32_t, r);
+  const uint32_t mag = b & 0x7fffffffu;
+  constexpr uint32_t DROP = DT == 1 ? 16u : 13u;                   // binary32 mantissa bits the 16-bit format drops
+  constexpr uint32_t LOW = (1u << DROP) - 1u, TIE = 1u << (DROP - 1u);
+  constexpr uint32_t LO = DT == 1 ? 0x00800000u : 0x38800000u;     // 2^-126 / 2^-14: smallest normal of the format
+  constexpr uint32_t HI = DT == 1 ? 0x7f000000u : 0x47000000u;     // 2^127 / 2^15: well below the overflow threshold
+  const bool safe = mag == 0u || (mag >= LO && mag < HI && (b & LOW) != TIE);
+  return safe ? f32_to_elem<DT>(r) : f64_to_elem<DT>(x);
+}
+
 // Packed 16-bit helpers.  A tile is kept in registers as the 16-bit patterns it was loaded with (two per register) and
 // widened where it is used: half the registers of a binary32 copy, which is what lets enough workgroups share a CU to
 // keep HBM busy.
@@ -148,6 +165,16 @@ template <> __device__ __forceinline__ uint32_t pack_round2<1>(float a, float b)
   typedef float f2 __attribute__((ext_vector_type(2)));
   const f2 v = {a, b};
   return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf2));   // v_cvt_pk_bf16_f32
+}
+// (int)y truncated toward zero, its low 8 bits written to byte B of acc: one instruction per element (the conversion's
+// sub-dword destination select) instead of a conversion plus shifts and ors.  Byte 0 clears the other three bytes, bytes
+// 1-3 keep them, so four calls in ascending order build a packed word without an initial value.
+template <int B>
+__device__ __forceinline__ void cvt_trunc_to_byte(uint32_t &acc, float y) {
+  if constexpr (B == 0) asm("v_cvt_i32_f32_sdwa %0, %1 dst_sel:BYTE_0 dst_unused:UNUSED_PAD src0_sel:DWORD" : "=v"(acc) : "v"(y));
+  else if constexpr (B == 1) asm("v_cvt_i32_f32_sdwa %0, %1 dst_sel:BYTE_1 dst_unused:UNUSED_PRESERVE src0_sel:DWORD" : "+v"(acc) : "v"(y));
+  else if constexpr (B == 2) asm("v_cvt_i32_f32_sdwa %0, %1 dst_sel:BYTE_2 dst_unused:UNUSED_PRESERVE src0_sel:DWORD" : "+v"(acc) : "v"(y));
+  else asm("v_cvt_i32_f32_sdwa %0, %1 dst_sel:BYTE_3 dst_unused:UNUSED_PRESERVE src0_sel:DWORD" : "+v"(acc) : "v"(y));
 }
 // Hides a register's value from the optimiser: placed between two passes over the packed tile, it keeps the compiler
 // from carrying the widened (binary32) copies of one pass over to the next, which would double the registers again.
@@ -327,7 +354,7 @@ __global__ __launch_bounds__(256) void pool_sim_quant_kernel(const uint16_t *__r
       for (int i = 0; i < RPP; i++) s += s_red[t_sb][i][t_col];
       // full blocks: the row count is a power of two, so the product with its reciprocal is the exact quotient
       const double mean = t_rows == BS ? s * (1.0 / BS) : s / (double)t_rows;
-      pool[((size_t)bh * nb + blk0 + t_sb) * D + t_col] = f64_to_elem<DT>(mean);
+      pool[((size_t)bh * nb + blk0 + t_sb) * D + t_col] = f64_to_elem_fast<DT>(mean);
     }
     long long g = 0;
     if (!sim_trivial) {
@@ -411,7 +438,7 @@ __global__ __launch_bounds__(256) void pool_sim_quant_kernel(const uint16_t *__r
       for (int p = sb * NP; p < (sb + 1) * NP; p++) {
         const int row = r + p * RPP;
         if (!decltype(check_rows)::value || row < rows_here) {
-          uint32_t pk[2] = {0, 0};
+          float y[8];
 #pragma unroll
           for (int j = 0; j < 4; j++) {
             float f[2];
@@ -419,14 +446,14 @@ __global__ __launch_bounds__(256) void pool_sim_quant_kernel(const uint16_t *__r
             unpack2<DT>(w[p][j], f[0], f[1]);
 #pragma unroll
             for (int h = 0; h < 2; h++) {
-              float y = divide(f[h]);
-              y = y + __builtin_copysignf(0.5f, y);   // +0.5 for y >= 0 (a -0 quotient truncates to 0 either way)
-              const int q = (int)y;   // truncation toward zero
-              const int e = 2 * j + h;
-              pk[e >> 2] |= ((uint32_t)q & 0xffu) << (8 * (e & 3));
+              const float t = divide(f[h]);
+              y[2 * j + h] = t + __builtin_copysignf(0.5f, t);   // +0.5 for t >= 0 (a -0 quotient truncates to 0 either way)
             }
           }
-          *(uint2 *)(qb + (size_t)row * D) = make_uint2(pk[0], pk[1]);
+          uint32_t pk0, pk1;                       // truncation toward zero, low 8 bits of element e into byte e % 4
+          cvt_trunc_to_byte<0>(pk0, y[0]); cvt_trunc_to_byte<1>(pk0, y[1]); cvt_trunc_to_byte<2>(pk0, y[2]); cvt_trunc_to_byte<3>(pk0, y[3]);
+          cvt_trunc_to_byte<0>(pk1, y[4]); cvt_trunc_to_byte<1>(pk1, y[5]); cvt_trunc_to_byte<2>(pk1, y[6]); cvt_trunc_to_byte<3>(pk1, y[7]);
+          *(uint2 *)(qb + (size_t)row * D) = make_uint2(pk0, pk1);
         }
       }
     };
@@ -504,23 +531,6 @@ __device__ __forceinline__ void emit_lut(FlagFn flag, int nk, int nkp, int32_t *
     lut_row[p] = v;
   }
   if (tid == 0) *valid_out = st.y;
-}
-
-// binary64 -> 16-bit pattern (round to nearest even) through binary32 where that provably gives the same bits: the
-// first rounding (to 24 bits) can only change the second one when it lands exactly on a rounding tie of the 16-bit
-// format, so every other value inside the format's normal range takes two hardware conversions instead of the 64-bit
-// integer arithmetic of f64_to_elem; ties, zero-range, subnormal and overflowing values go the exact way.
-template <int DT>
-__device__ __forceinline__ uint16_t f64_to_elem_fast(double x) {
-  const float r = (float)x;                                        // v_cvt_f32_f64
-  const uint32_t b = __builtin_bit_cast(uint32_t, r);
-  const uint32_t mag = b & 0x7fffffffu;
-  constexpr uint32_t DROP = DT == 1 ? 16u : 13u;                   // binary32 mantissa bits the 16-bit format drops
-  constexpr uint32_t LOW = (1u << DROP) - 1u, TIE = 1u << (DROP - 1u);
-  constexpr uint32_t LO = DT == 1 ? 0x00800000u : 0x38800000u;     // 2^-126 / 2^-14: smallest normal of the format
-  constexpr uint32_t HI = DT == 1 ? 0x7f000000u : 0x47000000u;     // 2^127 / 2^15: well below the overflow threshold
-  const bool safe = mag == 0u || (mag >= LO && mag < HI && (b & LOW) != TIE);
-  return safe ? f32_to_elem<DT>(r) : f64_to_elem<DT>(x);
 }
 
 // =============================================================================================
