@@ -38,7 +38,7 @@ __global__ __launch_bounds__(256) void v_absmax_kernel(const uint16_t *__restric
   // result is converted.
   typedef unsigned short u16x2_t __attribute__((ext_vector_type(2)));
   uint32_t mp[4] = {0, 0, 0, 0};
-#pragma unroll 8
+#pragma unroll 4
   for (int row = row0 + r; row < row1; row += RPP) {
     const uint4 q = *(const uint4 *)(base + (size_t)row * vs.sn);
     const uint32_t w[4] = {q.x, q.y, q.z, q.w};
