@@ -950,25 +950,25 @@ __global__ __launch_bounds__(64 * NW, (!DUAL && NW == 8) ? 2 : 1) void block_sel
       if (n < nk) {
         // top-k needs the n-th largest key only, not the order: build it bit by bit, the largest T with
         // #{key >= T} >= n.  Keys are distinct, probabilities are <= 1 (bits 31 and 30 of a key are clear) and
-        // bits 15 .. log2(NKP) are set in every real key (they hold 0xFFFF - column).
+        // bits 15 .. log2(NKP) are set in every real key (they hold 0xFFFF - column).  A candidate that exactly n keys
+        // reach selects the same set as the n-th largest key itself, so the search stops there.
         constexpr int LOW = 31 - __builtin_clz((unsigned)NKP);   // log2(NKP)
         uint32_t T = 0u;
-        auto at_least_n = [&](uint32_t cand) {
+        bool exact = false;                                      // wavefront-uniform
+        auto try_bit = [&](int bit) {
+          const uint32_t cand = T | (1u << bit);
           int cnt = 0;
 #pragma unroll
           for (int tt = 0; tt < EPL; tt++) cnt += __builtin_popcountll(__ballot(okey[tt] >= cand));
-          return cnt >= (int)n;
+          if (cnt >= (int)n) T = cand;
+          exact = cnt == (int)n;
         };
-#pragma unroll
-        for (int bit = 29; bit >= 16; bit--) {
-          const uint32_t cand = T | (1u << bit);
-          if (at_least_n(cand)) T = cand;
-        }
-        T |= 0xffffu & ~((1u << LOW) - 1u);
-#pragma unroll
-        for (int bit = LOW - 1; bit >= 0; bit--) {
-          const uint32_t cand = T | (1u << bit);
-          if (at_least_n(cand)) T = cand;
+#pragma unroll 1
+        for (int bit = 29; bit >= 16 && !exact; bit--) try_bit(bit);
+        if (!exact) {
+          T |= 0xffffu & ~((1u << LOW) - 1u);
+#pragma unroll 1
+          for (int bit = LOW - 1; bit >= 0 && !exact; bit--) try_bit(bit);
         }
         kth = T;
       }
