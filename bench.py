@@ -27,7 +27,7 @@ PEAK_HBM = 8.0e12
 # HBM-side bytes per launch of the attention kernel, measured with two rocprofv3 --pmc runs (FETCH_SIZE, WRITE_SIZE,
 # each scaled by what the same counter reads for a 1 GiB device copy: x2.0 and x1.0).  Only known for the workload
 # it was measured on.
-MEASURED_ATTN_TRAFFIC = {"cfg4": int((1.87 + 0.25) * 2 ** 30)}
+MEASURED_ATTN_TRAFFIC = {"cfg4": int((1.877 + 0.250) * 2 ** 30)}
 
 
 def parse():
