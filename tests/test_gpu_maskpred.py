@@ -139,6 +139,35 @@ def test_shared_reciprocal_division_is_ieee():
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_block_select_score_on_a_rounding_tie(dtype):
+    """A pooled score that lies just above a rounding tie of the 16-bit format, by less than binary32 resolves, must be
+    rounded from its exact value (up), not through binary32 (which lands on the tie and then rounds to even, down)."""
+    tag = tag_of(dtype)
+    B, H, nq, nk, D = 1, 1, 4, 8, 64
+    half_ulp = 0.25 if dtype == torch.bfloat16 else 2.0 ** -5       # half a unit in the last place at 64
+    q1, k1 = (0.5, 0.5) if dtype == torch.bfloat16 else (2.0 ** -3, 2.0 ** -2)
+    assert q1 * k1 == half_ulp
+    pq = torch.zeros((B, H, nq, D), dtype=dtype, device="cuda")
+    pk = torch.zeros((B, H, nk, D), dtype=dtype, device="cuda")
+    pq[..., 0], pq[..., 1], pq[..., 2] = 8.0, q1, 2.0 ** -10
+    pk[..., 0] = -8.0                                               # every other column: score -64
+    pk[0, 0, 2, :3] = torch.tensor([8.0, k1, 0.0], dtype=dtype)           # column 2: 64 + half_ulp exactly (tie -> 64)
+    pk[0, 0, 5, :3] = torch.tensor([8.0, k1, 2.0 ** -10], dtype=dtype)    # column 5: 2^-20 above the tie -> next value up
+    sq = torch.ones((B, H, nq), dtype=torch.bool, device="cuda")
+    sk = torch.ones((B, H, nk), dtype=torch.bool, device="cuda")
+    topk = torch.tensor([0.13], dtype=torch.float32, device="cuda")       # int(0.13 * 8) = 1 block per row
+    lut, valid, bmap = _lib.block_select(pq, sq, pk, sk, topk=topk, cdfthreshd=None, is_causal=False,
+                                         attention_sink=False, return_map=True)
+    ref_map = mp.block_map(to_np(pq), sq.cpu().numpy(), to_np(pk), sk.cpu().numpy(), tag, is_causal=False,
+                           topk=topk.cpu().numpy(), cdfthreshd=None, attention_sink=False)
+    want = np.zeros((B, H, nq, nk), bool)
+    want[..., 5] = True                                             # the larger score wins; a tie would go to column 2
+    assert np.array_equal(ref_map, want)
+    assert np.array_equal(bmap.cpu().numpy().astype(bool), want)
+    assert np.array_equal(valid.cpu().numpy(), np.ones((B, H, nq), np.int32))
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("thr_value", [-0.1, -1.0, 0.0, 0.3])
 def test_similarity_flag_on_degenerate_rows(dtype, thr_value):
     """Negative thresholds are decided without the normalised rows; the flag must still match the oracle on all-zero
