@@ -40,7 +40,7 @@ __global__ __launch_bounds__(256) void km_partial_kernel(const uint16_t *__restr
   for (int e = 0; e < 8; e++) acc[e] = 0.0;
 #pragma unroll 4
   for (int row = row0 + r; row < row1; row += RPP) {
-    const uint4 v = *(const uint4 *)(base + (size_t)row * ks.sn);
+    const uint4 v = load_stream_u4(base + (size_t)row * ks.sn);
     const uint32_t w[4] = {v.x, v.y, v.z, v.w};
 #pragma unroll
     for (int e = 0; e < 4; e++) {
@@ -231,7 +231,7 @@ __global__ __launch_bounds__(256) void pool_sim_quant_kernel(const uint16_t *__r
   {
     uint4 raw[NPT];
 #pragma unroll
-    for (int p = 0; p < NPT; p++) raw[p] = *(const uint4 *)(xb + (size_t)min(r + p * RPP, rows_here - 1) * xs.sn);
+    for (int p = 0; p < NPT; p++) raw[p] = load_stream_u4(xb + (size_t)min(r + p * RPP, rows_here - 1) * xs.sn);
 #pragma unroll
     for (int p = 0; p < NPT; p++) { w[p][0] = raw[p].x; w[p][1] = raw[p].y; w[p][2] = raw[p].z; w[p][3] = raw[p].w; }
   }

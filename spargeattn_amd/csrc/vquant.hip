@@ -40,7 +40,7 @@ __global__ __launch_bounds__(256) void v_absmax_kernel(const uint16_t *__restric
   uint32_t mp[4] = {0, 0, 0, 0};
 #pragma unroll 4
   for (int row = row0 + r; row < row1; row += RPP) {
-    const uint4 q = *(const uint4 *)(base + (size_t)row * vs.sn);
+    const uint4 q = load_stream_u4(base + (size_t)row * vs.sn);
     const uint32_t w[4] = {q.x, q.y, q.z, q.w};
 #pragma unroll
     for (int j = 0; j < 4; j++)
@@ -81,7 +81,7 @@ __global__ __launch_bounds__(256) void v_quant_kernel(const uint16_t *__restrict
   const int last_row = min(63, N - 1 - blk * 64);
   uint4 raw[NP];                     // every load is issued before the first use; rows beyond N re-read the last row
 #pragma unroll
-  for (int p = 0; p < NP; p++) raw[p] = *(const uint4 *)(base + (size_t)min(r + p * RPP, last_row) * vs.sn);
+  for (int p = 0; p < NP; p++) raw[p] = load_stream_u4(base + (size_t)min(r + p * RPP, last_row) * vs.sn);
 #pragma unroll
   for (int p = 0; p < NP; p++) {
     const int row = r + p * RPP;
