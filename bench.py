@@ -43,6 +43,9 @@ def parse():
     ap.add_argument("--copy-calibration", action="store_true",
                     help="run only a 1 GiB device-to-device copy (known traffic) - the reference point for scaling the "
                          "FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run")
+    ap.add_argument("--stream-calibration", action="store_true",
+                    help="run only the library's streaming probe (read-only, and read 2 bytes / write 1 byte per element) "
+                         "over a rotating 1 GiB footprint: the rates this machine gives the streaming kernels' shapes")
     ap.add_argument("--attn-only", action="store_true",
                     help="time only the attention kernel launches (for rocprofv3 runs of the dominant kernel)")
     return ap.parse_args()
@@ -84,6 +87,29 @@ def main():
             a.copy_(b)
         torch.cuda.synchronize()
         print(json.dumps({"copy_bytes_read": n, "copy_bytes_written": n}))
+        return
+
+    if args.stream_calibration:
+        torch.cuda.set_device(0)
+        n = 256 << 20                                   # bytes per launch; four regions rotate so that no cache can serve them
+        src = torch.ones(4 * n, dtype=torch.uint8, device="cuda")
+        dst = torch.empty(4 * (n // 2), dtype=torch.uint8, device="cuda")
+        sink = torch.zeros(1, dtype=torch.int32, device="cuda")
+        res = {}
+        for mode, name, moved in ((0, "read_nontemporal", n), (1, "read_plain", n), (2, "read2_write1", n + n // 2)):
+            def launch(i):
+                _lib.selftest_stream(src[(i % 4) * n:], dst[(i % 4) * (n // 2):], sink, n, mode)
+            for i in range(3):
+                launch(i)
+            evs = [torch.cuda.Event(enable_timing=True) for _ in range(21)]
+            evs[0].record()
+            for i in range(20):
+                launch(i)
+                evs[i + 1].record()
+            torch.cuda.synchronize()
+            us = sorted(evs[i].elapsed_time(evs[i + 1]) * 1e3 for i in range(20))[10]
+            res[name] = {"us_median": us, "bytes": moved, "TBps": moved / us / 1e6}
+        print(json.dumps({"stream_calibration": res}))
         return
 
     cfg = W.CONFIGS[args.config]

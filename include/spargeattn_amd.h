@@ -171,6 +171,12 @@ int spg_selftest_division(unsigned long long *counts, int n_divisors, unsigned i
  * saturate == 0: the bare v_cvt_pk_fp8_f32 instruction (NaN for |x| > 464), for documentation of the hardware. */
 int spg_selftest_fp8_pack(const float *x, uint8_t *codes, int n, int saturate, void *stream);
 
+/* ---- measurement aid (no counterpart in the reference): what the machine delivers for the access shapes of the
+ * streaming kernels, with nothing but the loads and stores.  mode 0: read `bytes` from src, 16 B per lane, non-temporal
+ * hint; mode 1: the same with plain loads; mode 2: read `bytes` (non-temporal) and write bytes/2 to dst (the 2-bytes-in,
+ * 1-byte-out shape of the quantisation kernels).  bytes is a multiple of 32768; sink is 4 writable bytes. */
+int spg_selftest_stream(const void *src, void *dst, void *sink, size_t bytes, int mode, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

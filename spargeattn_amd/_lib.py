@@ -36,6 +36,7 @@ SIGNATURES = {
     "spg_dense_attn_f16": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _f, _i, _vp]),
     "spg_selftest_division": (_i, [_vp, _i, ctypes.c_uint, _vp]),
     "spg_selftest_fp8_pack": (_i, [_vp, _vp, _i, _i, _vp]),
+    "spg_selftest_stream": (_i, [_vp, _vp, _vp, ctypes.c_size_t, _i, _vp]),
 }
 
 _lib = None
@@ -314,6 +315,14 @@ def selftest_fp8_pack(x, saturate=True):
     codes = torch.empty(x.numel(), dtype=torch.uint8, device=x.device)
     _check(load().spg_selftest_fp8_pack(_p(x), _p(codes), x.numel(), int(bool(saturate)), _stream()))
     return codes.view(x.shape)
+
+
+def selftest_stream(src, dst, sink, nbytes, mode):
+    """Launches the streaming probe once: mode 0 / 1 read nbytes of src (non-temporal / plain loads), mode 2 reads nbytes
+    and writes nbytes / 2 to dst."""
+    _dev(src, sink)
+    _check(load().spg_selftest_stream(_p(src), _p(dst) if dst is not None else None, _p(sink), int(nbytes), int(mode),
+                                      _stream()))
 
 
 def selftest_division(n_divisors, seed=1):

@@ -165,6 +165,17 @@ int spg_selftest_fp8_pack(const float *x, uint8_t *codes, int n, int saturate, v
   return check_launch(fn, hipSuccess);
 }
 
+int spg_selftest_stream(const void *src, void *dst, void *sink, size_t bytes, int mode, void *stream) {
+  const char *fn = "spg_selftest_stream";
+  if (bytes == 0 || bytes % 32768 != 0 || bytes / 32768 > 0x7fffffffull)
+    return fail(SPG_ERR_INVALID, "%s: bytes must be a positive multiple of 32768 (got %zu)", fn, bytes);
+  if (mode < 0 || mode > 2) return fail(SPG_ERR_INVALID, "%s: mode must be 0, 1 or 2 (got %d)", fn, mode);
+  SPG_NONNULL(fn, src); SPG_NONNULL(fn, sink);
+  if (mode == 2) SPG_NONNULL(fn, dst);
+  spg::launch_stream_probe(src, dst, sink, bytes, mode, (hipStream_t)stream);
+  return check_launch(fn, hipSuccess);
+}
+
 int spg_v_quant_fp8(const void *v, const int64_t *v_strides, uint8_t *v8, float *v_scale, int B, int H, int N, int D, int dtype, void *stream) {
   const char *fn = "spg_v_quant_fp8";
   SPG_TRY(check_shape(fn, B, H, N, D));

@@ -41,6 +41,7 @@ hipError_t launch_block_sparse_attn(const int8_t *q8, const int8_t *k8, const ui
                                     int Hkv, int N, int Nk, int D, float sm_scale, int is_causal, int pv_mode,
                                     int32_t *pv_count, hipStream_t st);
 void launch_fp8_pack_selftest(const float *x, uint8_t *codes, int n, int saturate, hipStream_t st);
+void launch_stream_probe(const void *src, void *dst, void *sink, size_t bytes, int mode, hipStream_t st);
 
 hipError_t launch_dense_attn_f16(const void *q, const void *k, const void *v, void *out, int B, int H, int N, int D,
                                  float sm_scale, int is_causal, hipStream_t st);
