@@ -124,7 +124,7 @@ __global__ __launch_bounds__(256) void v_tiles_f16_kernel(const uint16_t *__rest
   const int last_row = min(63, N - 1 - blk * 64);
   uint4 raw[NP];
 #pragma unroll
-  for (int p = 0; p < NP; p++) raw[p] = *(const uint4 *)(base + (size_t)min(r + p * RPP, last_row) * vs.sn);
+  for (int p = 0; p < NP; p++) raw[p] = load_stream_u4(base + (size_t)min(r + p * RPP, last_row) * vs.sn);
 #pragma unroll
   for (int p = 0; p < NP; p++) {
     const int row = r + p * RPP;
