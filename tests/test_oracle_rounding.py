@@ -111,3 +111,50 @@ def test_fp32_subtraction_then_rne_equals_single_rounding():
         b2 = R.round_to(p2 * 2.0 ** -rng.integers(8, 26, 100000), tag).astype(np.float64)
         assert np.array_equal(R.round_to(a2 - b2, tag),
                               R.round_to((a2.astype(np.float32) - b2.astype(np.float32)).astype(np.float64), tag))
+
+
+def _safe_for_two_step(r32, tag):
+    """The predicate of the kernels' binary64 -> 16-bit shortcut (csrc/maskpred.hip, f64_to_elem_fast): the binary32 image
+    is zero, or inside the 16-bit format's normal range and not exactly on one of its rounding ties."""
+    b = np.ascontiguousarray(r32, dtype=np.float32).view(np.uint32)
+    mag = b & np.uint32(0x7fffffff)
+    drop = 16 if tag == R.BF16 else 13
+    low, tie = np.uint32((1 << drop) - 1), np.uint32(1 << (drop - 1))
+    lo = np.uint32(0x00800000 if tag == R.BF16 else 0x38800000)
+    hi = np.uint32(0x7f000000 if tag == R.BF16 else 0x47000000)
+    return (mag == 0) | ((mag >= lo) & (mag < hi) & ((b & low) != tie))
+
+
+def test_binary64_to_16_bits_through_binary32_where_the_kernels_take_that_way():
+    """Rounding a binary64 value to binary32 first changes its rounding to a 16-bit format only when the binary32 image
+    lands exactly on a tie of that format: wherever the kernels' predicate holds, both ways give the same bits - also
+    for a value two units in the last place away (the reciprocal-based probabilities)."""
+    rng = np.random.default_rng(4)
+    for tag in (R.BF16, R.FP16):
+        drop = 16 if tag == R.BF16 else 13
+        # random magnitudes over the whole normal range, values sitting on and next to ties, next to binade edges
+        e = rng.integers(-14, 15, size=400000) if tag == R.FP16 else rng.integers(-126, 127, size=400000)
+        x = np.ldexp(1.0 + rng.random(400000), e) * rng.choice([-1.0, 1.0], size=400000)
+        grid = np.ldexp(1.0 + rng.integers(0, 1 << (23 - drop), size=200000) * 2.0 ** -(23 - drop),
+                        rng.integers(-10, 10, size=200000))                  # values of the 16-bit format
+        ulp = np.ldexp(1.0, np.floor(np.log2(grid)).astype(np.int64) - (23 - drop))
+        tie = grid + 0.5 * ulp
+        near = np.concatenate([tie, tie * (1 + 2.0 ** -30), tie * (1 - 2.0 ** -30), tie * (1 + 2.0 ** -52),
+                               tie * (1 - 2.0 ** -52), tie + 2.0 ** -24 * grid, grid * (1 - 2.0 ** -40),
+                               grid * (1 + 2.0 ** -40)])
+        for vals, least in ((x, 0.95), (near, 0.25)):
+            r32 = vals.astype(np.float32)
+            safe = _safe_for_two_step(r32, tag)
+            assert safe.mean() > least
+            direct = R.bits16(R.round_to(vals, tag), tag)
+            two_step = R.bits16(R.round_to(r32.astype(np.float64), tag), tag)
+            assert np.array_equal(direct[safe], two_step[safe])
+            # a neighbour within two units in the last place of binary64 rounds like the value itself
+            for k in (-2, 2):
+                nb = (vals.view(np.int64) + k).view(np.float64)
+                assert np.array_equal(R.bits16(R.round_to(nb, tag), tag)[safe], two_step[safe])
+        # and the predicate is not vacuous: on the ties themselves the two ways differ somewhere
+        r32 = (tie * (1 + 2.0 ** -30)).astype(np.float32)
+        assert (~_safe_for_two_step(r32, tag)).any()
+        assert not np.array_equal(R.bits16(R.round_to(tie * (1 + 2.0 ** -30), tag), tag),
+                                  R.bits16(R.round_to(r32.astype(np.float64), tag), tag))
