@@ -177,6 +177,12 @@ int spg_selftest_fp8_pack(const float *x, uint8_t *codes, int n, int saturate, v
  * 1-byte-out shape of the quantisation kernels).  bytes is a multiple of 32768; sink is 4 writable bytes. */
 int spg_selftest_stream(const void *src, void *dst, void *sink, size_t bytes, int mode, void *stream);
 
+/* ---- measurement aid (no counterpart in the reference): how matrix and vector instructions share a SIMD.  Every
+ * wavefront of `blocks` workgroups (256 threads) repeats 4 * reps times "one MFMA, then nv independent v_add_f32" with two
+ * accumulator chains.  kind 0: v_mfma_i32_32x32x32_i8, 1: v_mfma_f32_32x32x64_f8f6f4, 2: v_mfma_f32_32x32x16_f16;
+ * nv in {0, 8, 16, 32, 64}; out: blocks * 256 floats. */
+int spg_selftest_issue(float *out, int kind, int nv, int reps, int blocks, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -37,6 +37,7 @@ SIGNATURES = {
     "spg_selftest_division": (_i, [_vp, _i, ctypes.c_uint, _vp]),
     "spg_selftest_fp8_pack": (_i, [_vp, _vp, _i, _i, _vp]),
     "spg_selftest_stream": (_i, [_vp, _vp, _vp, ctypes.c_size_t, _i, _vp]),
+    "spg_selftest_issue": (_i, [_vp, _i, _i, _i, _i, _vp]),
 }
 
 _lib = None
@@ -323,6 +324,13 @@ def selftest_stream(src, dst, sink, nbytes, mode):
     _dev(src, sink)
     _check(load().spg_selftest_stream(_p(src), _p(dst) if dst is not None else None, _p(sink), int(nbytes), int(mode),
                                       _stream()))
+
+
+def selftest_issue(out, kind, nv, reps, blocks):
+    """Launches the issue probe once: every wavefront repeats 4 * reps times one MFMA of `kind` + nv vector adds."""
+    _dev(out)
+    assert out.dtype == torch.float32 and out.numel() >= blocks * 256
+    _check(load().spg_selftest_issue(_p(out), int(kind), int(nv), int(reps), int(blocks), _stream()))
 
 
 def selftest_division(n_divisors, seed=1):

@@ -176,6 +176,15 @@ int spg_selftest_stream(const void *src, void *dst, void *sink, size_t bytes, in
   return check_launch(fn, hipSuccess);
 }
 
+int spg_selftest_issue(float *out, int kind, int nv, int reps, int blocks, void *stream) {
+  const char *fn = "spg_selftest_issue";
+  if (reps <= 0 || blocks <= 0) return fail(SPG_ERR_INVALID, "%s: reps and blocks must be positive", fn);
+  SPG_NONNULL(fn, out);
+  if (!spg::launch_issue_probe(out, kind, nv, reps, blocks, (hipStream_t)stream))
+    return fail(SPG_ERR_INVALID, "%s: kind must be 0, 1 or 2 and nv one of 0, 8, 16, 32, 64 (got %d, %d)", fn, kind, nv);
+  return check_launch(fn, hipSuccess);
+}
+
 int spg_v_quant_fp8(const void *v, const int64_t *v_strides, uint8_t *v8, float *v_scale, int B, int H, int N, int D, int dtype, void *stream) {
   const char *fn = "spg_v_quant_fp8";
   SPG_TRY(check_shape(fn, B, H, N, D));

@@ -42,6 +42,7 @@ hipError_t launch_block_sparse_attn(const int8_t *q8, const int8_t *k8, const ui
                                     int32_t *pv_count, hipStream_t st);
 void launch_fp8_pack_selftest(const float *x, uint8_t *codes, int n, int saturate, hipStream_t st);
 void launch_stream_probe(const void *src, void *dst, void *sink, size_t bytes, int mode, hipStream_t st);
+bool launch_issue_probe(float *out, int kind, int nv, int reps, int blocks, hipStream_t st);
 
 hipError_t launch_dense_attn_f16(const void *q, const void *k, const void *v, void *out, int B, int H, int N, int D,
                                  float sm_scale, int is_causal, hipStream_t st);

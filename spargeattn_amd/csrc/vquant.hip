@@ -190,33 +190,4 @@ void launch_v_tiles_f16(const void *v, Strides vs, void *vt, int B, int H, int N
   else         { if (dtype == 0) v_tiles_f16_kernel<128, 0><<<grid, 256, 0, st>>>(vp, vs, H, op, N, nk); else v_tiles_f16_kernel<128, 1><<<grid, 256, 0, st>>>(vp, vs, H, op, N, nk); }
 }
 
-// Streaming probe: what this machine delivers for the access shapes of the kernels above, measured with nothing but the
-// loads and stores.  mode 0: read 16 B per lane with the non-temporal hint; mode 1: the same with plain loads; mode 2:
-// read 16 B (non-temporal) and write 8 B per lane (the 2-bytes-in, 1-byte-out shape of the quantisation kernels).  One
-// workgroup per 32 KiB of input.
-template <int MODE>
-__global__ __launch_bounds__(256) void stream_probe_kernel(const uint4 *__restrict__ src, uint2 *__restrict__ dst,
-                                                           uint32_t *__restrict__ sink) {
-  const size_t base = (size_t)blockIdx.x * 2048;
-  uint4 v[8];
-#pragma unroll
-  for (int u = 0; u < 8; u++) {
-    const uint4 *a = src + base + threadIdx.x + u * 256;
-    v[u] = MODE == 1 ? *a : load_stream_u4(a);
-  }
-  uint32_t acc = 0;
-#pragma unroll
-  for (int u = 0; u < 8; u++) {
-    if constexpr (MODE == 2) dst[base + threadIdx.x + u * 256] = make_uint2(v[u].x ^ v[u].y, v[u].z ^ v[u].w);
-    else acc ^= v[u].x ^ v[u].y ^ v[u].z ^ v[u].w;
-  }
-  if (MODE != 2 && acc == 0x9e3779b9u) sink[0] = acc;      // keeps the loads alive; practically never true
-}
-void launch_stream_probe(const void *src, void *dst, void *sink, size_t bytes, int mode, hipStream_t st) {
-  const int grid = (int)(bytes / 32768);
-  if (mode == 0) stream_probe_kernel<0><<<grid, 256, 0, st>>>((const uint4 *)src, (uint2 *)dst, (uint32_t *)sink);
-  else if (mode == 1) stream_probe_kernel<1><<<grid, 256, 0, st>>>((const uint4 *)src, (uint2 *)dst, (uint32_t *)sink);
-  else stream_probe_kernel<2><<<grid, 256, 0, st>>>((const uint4 *)src, (uint2 *)dst, (uint32_t *)sink);
-}
-
 }  // namespace spg

@@ -19,7 +19,7 @@ def _declared():
 def test_header_declares_the_stages():
     names = _declared()
     for want in ("spg_km_mean", "spg_pool_sim_quant", "spg_block_select", "spg_map_to_lut", "spg_v_quant_fp8",
-                 "spg_block_sparse_attn", "spg_block_sparse_attn_f16v", "spg_v_tiles_f16", "spg_dense_attn_f16", "spg_selftest_division", "spg_selftest_fp8_pack", "spg_selftest_stream", "spg_last_error", "spg_version"):
+                 "spg_block_sparse_attn", "spg_block_sparse_attn_f16v", "spg_v_tiles_f16", "spg_dense_attn_f16", "spg_selftest_division", "spg_selftest_fp8_pack", "spg_selftest_stream", "spg_selftest_issue", "spg_last_error", "spg_version"):
         assert want in names
 
 

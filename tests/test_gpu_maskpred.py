@@ -264,3 +264,17 @@ def test_stream_probe_copies_what_it_reads():
     assert torch.equal(dst, want)
     with pytest.raises(ValueError):
         _lib.selftest_stream(src, dst, sink, 1000, 2)
+
+
+def test_issue_probe_runs_and_rejects_unknown_shapes():
+    """The issue probe (a measurement aid) launches for every MFMA kind and add count it advertises."""
+    out = torch.full((4 * 256,), float("nan"), dtype=torch.float32, device="cuda")
+    for kind in (0, 1, 2):
+        for nv in (0, 8, 16, 32, 64):
+            _lib.selftest_issue(out, kind, nv, 3, 4)
+    torch.cuda.synchronize()
+    assert torch.isfinite(out).all()
+    with pytest.raises(ValueError):
+        _lib.selftest_issue(out, 3, 8, 3, 4)
+    with pytest.raises(ValueError):
+        _lib.selftest_issue(out, 0, 7, 3, 4)
