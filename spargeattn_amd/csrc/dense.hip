@@ -37,14 +37,15 @@ __device__ __forceinline__ uint32_t dense_k_swz(uint32_t row) {
 }
 
 template <int D, int NW>
-__global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void dense_attn_f16_kernel(const DenseParams p) {
+__global__ __launch_bounds__(64 * NW, 2) void dense_attn_f16_kernel(const DenseParams p) {
   constexpr int KS = D / 16;          // k-steps of QK^T
   constexpr int NDT = D / 32;         // output channel tiles
   constexpr int TILE = 64 * D * 2;    // bytes of one K tile and of one V^T tile
   constexpr int CPR = D / 8;          // 16-byte chunks per K row
   constexpr int QROWS = 32 * NW;      // query rows per workgroup
   constexpr int BPQ = QROWS / 64;     // key blocks per query tile on the diagonal
-  constexpr int WL = TILE / (1024 * NW);   // global_load_lds instructions per wavefront per tile
+  constexpr int PIECES = TILE / 1024; // 1 KiB pieces (one global_load_lds instruction each) per tile
+  constexpr int WL = (PIECES + NW - 1) / NW;   // pieces per wavefront per tile, at most (the last wavefronts may take fewer)
   constexpr int NBUF = 2;
   __shared__ __align__(1024) unsigned char smem[NBUF * 2 * TILE];   // K ring | V^T ring
   const uint32_t lds_k0 = (uint32_t)(size_t)(__attribute__((address_space(3))) unsigned char *)smem;
@@ -78,37 +79,41 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void dense_attn_f16_kerne
   // are masked below and their V rows are zero.
   typedef __attribute__((address_space(3))) void *lds_ptr_t;
   typedef const __attribute__((address_space(1))) void *glb_ptr_t;
+  // wavefront w takes pieces [first, first + npieces): the first PIECES % NW wavefronts take one piece more
+  constexpr int BASE = PIECES / NW, EXTRA = PIECES % NW;
+  const int npieces = BASE + (wave < EXTRA ? 1 : 0);
+  const int first = BASE * wave + min(wave, EXTRA);
   uint32_t k_off[WL];
 #pragma unroll
   for (int u = 0; u < WL; u++) {
-    const uint32_t pos = (uint32_t)(64 * (WL * wave + u) + lane);
+    const uint32_t pos = (uint32_t)(64 * (first + u) + lane);
     const uint32_t row = pos / CPR, slot = pos % CPR;
     k_off[u] = row * (D * 2) + ((slot ^ dense_k_swz<D>(row)) * 16u);
   }
-  const uint32_t v_off = (uint32_t)(WL * 1024 * wave + 16 * lane);
+  const uint32_t v_off = (uint32_t)(1024 * first + 16 * lane);
   const int last_partial_blk = (N % 64) ? p.nk - 1 : -1;
   auto load_tiles = [&](int blk, int slot) __attribute__((always_inline)) {
     const unsigned char *kb = kbase + (size_t)blk * TILE;
     const unsigned char *vb = vbase + (size_t)blk * TILE;
-    unsigned char *lk = smem + slot * TILE + WL * wave * 1024;
-    unsigned char *lv = smem + (NBUF + slot) * TILE + WL * wave * 1024;
+    unsigned char *lk = smem + slot * TILE + first * 1024;
+    unsigned char *lv = smem + (NBUF + slot) * TILE + first * 1024;
     if (blk != last_partial_blk) {
 #pragma unroll
       for (int u = 0; u < WL; u++)
-        __builtin_amdgcn_global_load_lds((glb_ptr_t)(kb + k_off[u]), (lds_ptr_t)(lk + u * 1024), 16, 0, 0);
+        if (u < npieces) __builtin_amdgcn_global_load_lds((glb_ptr_t)(kb + k_off[u]), (lds_ptr_t)(lk + u * 1024), 16, 0, 0);
     } else {
       const uint32_t rows_ok = (uint32_t)(N - blk * 64);
 #pragma unroll
       for (int u = 0; u < WL; u++) {
-        const uint32_t pos = (uint32_t)(64 * (WL * wave + u) + lane);
+        const uint32_t pos = (uint32_t)(64 * (first + u) + lane);
         const uint32_t row = min(pos / CPR, rows_ok - 1), slot_ = pos % CPR;
         const uint32_t ko = row * (D * 2) + ((slot_ ^ dense_k_swz<D>(pos / CPR)) * 16u);
-        __builtin_amdgcn_global_load_lds((glb_ptr_t)(kb + ko), (lds_ptr_t)(lk + u * 1024), 16, 0, 0);
+        if (u < npieces) __builtin_amdgcn_global_load_lds((glb_ptr_t)(kb + ko), (lds_ptr_t)(lk + u * 1024), 16, 0, 0);
       }
     }
 #pragma unroll
     for (int u = 0; u < WL; u++)
-      __builtin_amdgcn_global_load_lds((glb_ptr_t)(vb + v_off + u * 1024), (lds_ptr_t)(lv + u * 1024), 16, 0, 0);
+      if (u < npieces) __builtin_amdgcn_global_load_lds((glb_ptr_t)(vb + v_off + u * 1024), (lds_ptr_t)(lv + u * 1024), 16, 0, 0);
   };
 
   // MFMA row i of key tile kt carries key 32*((i>>2)&1) + 16*kt + 4*(i>>3) + (i&3): after S^T, register e of tile kt in
@@ -116,9 +121,9 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void dense_attn_f16_kerne
   // have the same swizzle, so tile 1's operand sits 16 rows after tile 0's.
   const uint32_t krow0 = (uint32_t)(32 * ((r >> 2) & 1) + 4 * (r >> 3) + (r & 3));
   const uint32_t ksw = dense_k_swz<D>(krow0);
-  uint32_t kaddr[KS];
-#pragma unroll
-  for (int ks = 0; ks < KS; ks++) kaddr[ks] = lds_k0 + krow0 * (D * 2) + ((((uint32_t)(2 * ks + hh)) ^ ksw) * 16u);
+  // K operand of k-step ks: chunk (2 ks + hh) ^ ksw of row krow0, i.e. byte k_rd_base + ((32 ks) ^ k_rd_x)
+  const uint32_t k_rd_base = lds_k0 + krow0 * (D * 2) + (((uint32_t)hh ^ ksw) & 1u) * 16u;
+  const uint32_t k_rd_x = (ksw & ~1u) * 16u;
   // V^T operand of key step s: chunk (4 hh + s) ^ ((r >> 1) & 7) of the 128-byte row r (+ 32 dt): va ^ (16 s)
   const uint32_t va0 = lds_v0 + (uint32_t)(r * 128 + (((4 * hh) ^ ((r >> 1) & 7)) * 16));
 
@@ -146,25 +151,20 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void dense_attn_f16_kerne
 #pragma unroll
     for (int e = 0; e < 16; e++) { S0[e] = 0.f; S1[e] = 0.f; }
     {
-      constexpr int HK = KS / 2;
-      v4i a0[KS], a1[KS];
+      // one k-step (two reads) in flight while the previous one multiplies: two small operand buffers
+      v4i a0[2], a1[2];
+      lds_read_2x128<SO, SO + 16 * D * 2>(a0[0], a1[0], k_rd_base + k_rd_x);
 #pragma unroll
-      for (int ks = 0; ks < HK; ks++) lds_read_2x128<SO, SO + 16 * D * 2>(a0[ks], a1[ks], kaddr[ks]);
-      if constexpr (HK == 4) { lds_wait4(a0[0], a1[0], a0[1], a1[1]); lds_wait4(a0[2], a1[2], a0[3], a1[3]); }
-      else lds_wait4(a0[0], a1[0], a0[1], a1[1]);
-#pragma unroll
-      for (int ks = HK; ks < KS; ks++) lds_read_2x128<SO, SO + 16 * D * 2>(a0[ks], a1[ks], kaddr[ks]);
-#pragma unroll
-      for (int ks = 0; ks < HK; ks++) {
-        S0 = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(v8h, a0[ks]), qreg[ks], S0, 0, 0, 0);
-        S1 = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(v8h, a1[ks]), qreg[ks], S1, 0, 0, 0);
-      }
-      if constexpr (HK == 4) { lds_wait4(a0[4], a1[4], a0[5], a1[5]); lds_wait4(a0[6], a1[6], a0[7], a1[7]); }
-      else lds_wait4(a0[2], a1[2], a0[3], a1[3]);
-#pragma unroll
-      for (int ks = HK; ks < KS; ks++) {
-        S0 = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(v8h, a0[ks]), qreg[ks], S0, 0, 0, 0);
-        S1 = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(v8h, a1[ks]), qreg[ks], S1, 0, 0, 0);
+      for (int ks = 0; ks < KS; ks++) {
+        const int cur = ks & 1, nxt = cur ^ 1;
+        if (ks + 1 < KS) {
+          lds_read_2x128<SO, SO + 16 * D * 2>(a0[nxt], a1[nxt], k_rd_base + ((uint32_t)(32 * (ks + 1)) ^ k_rd_x));
+          asm volatile("s_waitcnt lgkmcnt(2)" : "+v"(a0[cur]), "+v"(a1[cur]));   // all but the two reads just issued
+        } else {
+          lds_wait2(a0[cur], a1[cur]);
+        }
+        S0 = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(v8h, a0[cur]), qreg[ks], S0, 0, 0, 0);
+        S1 = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(v8h, a1[cur]), qreg[ks], S1, 0, 0, 0);
       }
     }
 
@@ -213,34 +213,30 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void dense_attn_f16_kerne
         pb[s4][j + 1] = (_Float16)h2[1];
       }
 
-    // ---- O^T += V^T . P^T: key steps 0,1 are read first; steps 2,3 are in flight while 0,1 multiply
+    // ---- O^T += V^T . P^T: the reads of key step s + 1 are in flight while step s multiplies
     {
       const uint32_t va = va0;
-      v4i t[4][NDT];
+      v4i t[2][NDT];
+      auto read_v = [&](int buf, int s4) __attribute__((always_inline)) {
+        lds_read_2x128<SO, SO + 4096>(t[buf][0], t[buf][1], va ^ (uint32_t)(16 * s4));
+        if constexpr (NDT == 4) lds_read_2x128<SO + 8192, SO + 12288>(t[buf][2], t[buf][3], va ^ (uint32_t)(16 * s4));
+      };
+      read_v(0, 0);
 #pragma unroll
-      for (int s4 = 0; s4 < 2; s4++) {
-        lds_read_2x128<SO, SO + 4096>(t[s4][0], t[s4][1], va ^ (uint32_t)(16 * s4));
-        if constexpr (NDT == 4) lds_read_2x128<SO + 8192, SO + 12288>(t[s4][2], t[s4][3], va ^ (uint32_t)(16 * s4));
-      }
-      if constexpr (NDT == 4) { lds_wait4(t[0][0], t[0][1], t[0][2], t[0][3]); lds_wait4(t[1][0], t[1][1], t[1][2], t[1][3]); }
-      else { lds_wait4(t[0][0], t[0][1], t[1][0], t[1][1]); }
-#pragma unroll
-      for (int s4 = 2; s4 < 4; s4++) {
-        lds_read_2x128<SO, SO + 4096>(t[s4][0], t[s4][1], va ^ (uint32_t)(16 * s4));
-        if constexpr (NDT == 4) lds_read_2x128<SO + 8192, SO + 12288>(t[s4][2], t[s4][3], va ^ (uint32_t)(16 * s4));
-      }
-#pragma unroll
-      for (int s4 = 0; s4 < 2; s4++)
-#pragma unroll
-        for (int dt = 0; dt < NDT; dt++)
-          O[dt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(v8h, t[s4][dt]), pb[s4], O[dt], 0, 0, 0);
-      if constexpr (NDT == 4) { lds_wait4(t[2][0], t[2][1], t[2][2], t[2][3]); lds_wait4(t[3][0], t[3][1], t[3][2], t[3][3]); }
-      else { lds_wait4(t[2][0], t[2][1], t[3][0], t[3][1]); }
-#pragma unroll
-      for (int s4 = 2; s4 < 4; s4++)
+      for (int s4 = 0; s4 < 4; s4++) {
+        const int cur = s4 & 1, nxt = cur ^ 1;
+        if (s4 + 1 < 4) {
+          read_v(nxt, s4 + 1);
+          if constexpr (NDT == 4) asm volatile("s_waitcnt lgkmcnt(4)" : "+v"(t[cur][0]), "+v"(t[cur][1]), "+v"(t[cur][2]), "+v"(t[cur][3]));
+          else asm volatile("s_waitcnt lgkmcnt(2)" : "+v"(t[cur][0]), "+v"(t[cur][1]));
+        } else {
+          if constexpr (NDT == 4) lds_wait4(t[cur][0], t[cur][1], t[cur][2], t[cur][3]);
+          else lds_wait2(t[cur][0], t[cur][1]);
+        }
 #pragma unroll
         for (int dt = 0; dt < NDT; dt++)
-          O[dt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(v8h, t[s4][dt]), pb[s4], O[dt], 0, 0, 0);
+          O[dt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(v8h, t[cur][dt]), pb[s4], O[dt], 0, 0, 0);
+      }
     }
     __builtin_amdgcn_s_waitcnt(0x0F70);   // this wavefront's share of block blk+1's tiles has landed in LDS
     __syncthreads();                      // block blk+1's tiles are complete; every wavefront is done with block blk's
@@ -277,7 +273,8 @@ hipError_t launch_dense_attn_f16(const void *q, const void *k, const void *vt, v
                                  float sm_scale, int is_causal, hipStream_t st) {
   DenseParams p;
   p.q = (const uint16_t *)q; p.k = (const uint16_t *)k; p.vt = (const uint16_t *)vt; p.out = (uint16_t *)out;
-  // wavefronts (32 query rows each) per workgroup: 8 share a tile pair at D = 128 (one 64 KiB ring per CU), 4 at D = 64
+  // wavefronts (32 query rows each) per workgroup: 6 share a tile pair at D = 128 (two 64 KiB rings per CU, three
+  // wavefronts per SIMD at 168 registers), 4 at D = 64
   const int NW = D == 64 ? 4 : 8;
   p.B = B; p.H = H; p.N = N; p.nq = (N + 32 * NW - 1) / (32 * NW); p.nk = (N + 63) / 64;
   p.sm_scale_log2 = sm_scale * 1.44269504088896340736f;
