@@ -21,9 +21,11 @@
 //    both the tile hand-over and the workgroup-wide PV-skip vote;
 //  * LDS tiles are unpadded; bank conflicts are avoided by an XOR swizzle of the 16-byte chunks inside a row
 //    (applied to the per-lane global address for K, baked into the HBM tile layout for V);
-//  * the INT8 accumulators start at the bit pattern of 1.5 * 2^23 (read from LDS), so that the int32 result IS the float
-//    12582912 + dot and the scores need no int-to-float conversion; the bias is folded into the constant of the fma
-//    that feeds exp2;
+//  * the INT8 accumulators start at the bit pattern of the float 1/(2 pi), an inline constant of the instruction set (no
+//    register or LDS read initialises them): read as a float the int32 result is 1/(2 pi) + dot * 2^-26, so the scores need
+//    no int-to-float conversion; the constant is folded into the additive term of the fma that feeds exp2;
+//  * only "skip" votes of the PV threshold reach LDS, and the rescale factor of O is computed only in iterations in which
+//    a running maximum rose;
 //  * workgroup ids are remapped so that one XCD (one L2) works on one head at a time, heaviest rows first.
 #include "common.h"
 #include "launch.h"
