@@ -1,11 +1,13 @@
 // Sparse-mask prediction and INT8 Q/K quantisation for gfx950.
 //
-// Kernels (one 16-byte load per lane, 64-lane wavefront reductions; the K mean streams at HBM speed, the other
-// kernels move only their algorithmic bytes but are bound by the exact arithmetic they carry):
+// Kernels (one 16-byte load per lane, 64-lane wavefront reductions; the K mean and the pooling / quantisation kernels run
+// at the rates the machine gives a bare read and a bare 2-bytes-in / 1-byte-out copy, the selection is bound by the
+// exact arithmetic it carries):
 //   km_partial / km_final      K column mean                          (spas_sage_attn/core.py:119-120)
 //   pool_sim_quant             pool + self-similarity + INT8 quant    (spas_sage_attn/utils.py:161-214, 89-159)
-//   block_select_wave / block_select   compressed QK^T softmax, top-k / CDF selection, block map, delta LUT: one
-//                              wavefront per row with the row in registers (nk <= 2048), one workgroup per row beyond
+//   block_select_wave / block_select   compressed QK^T softmax, top-k / CDF selection, block map, delta LUT: pooled
+//                              scores on the binary64 matrix unit and one wavefront per row with the row in registers
+//                              (nk <= 2048), one workgroup per row beyond
 //                                                                     (spas_sage_attn/utils.py:386-420, 54-87, 282-316)
 //   map_to_lut                 user block mask -> LUT                 (spas_sage_attn/utils.py:54-87)
 //
