@@ -43,13 +43,6 @@ def parse():
     ap.add_argument("--copy-calibration", action="store_true",
                     help="run only a 1 GiB device-to-device copy (known traffic) - the reference point for scaling the "
                          "FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run")
-    ap.add_argument("--stream-calibration", action="store_true",
-                    help="run only the library's streaming probe (read-only, and read 2 bytes / write 1 byte per element) "
-                         "over a rotating 1 GiB footprint: the rates this machine gives the streaming kernels' shapes")
-    ap.add_argument("--issue-calibration", action="store_true",
-                    help="run only the library's issue probe: time per 'one MFMA + NV vector adds' per SIMD at three "
-                         "wavefronts per SIMD, for the MFMA shapes of the attention kernels - how far vector instructions "
-                         "hide behind the matrix pipe on this machine")
     ap.add_argument("--attn-only", action="store_true",
                     help="time only the attention kernel launches (for rocprofv3 runs of the dominant kernel)")
     return ap.parse_args()
@@ -91,55 +84,6 @@ def main():
             a.copy_(b)
         torch.cuda.synchronize()
         print(json.dumps({"copy_bytes_read": n, "copy_bytes_written": n}))
-        return
-
-    if args.stream_calibration:
-        torch.cuda.set_device(0)
-        n = 256 << 20                                   # bytes per launch; four regions rotate so that no cache can serve them
-        src = torch.ones(4 * n, dtype=torch.uint8, device="cuda")
-        dst = torch.empty(4 * (n // 2), dtype=torch.uint8, device="cuda")
-        sink = torch.zeros(1, dtype=torch.int32, device="cuda")
-        res = {}
-        for mode, name, moved in ((0, "read_nontemporal", n), (1, "read_plain", n), (2, "read2_write1", n + n // 2)):
-            def launch(i):
-                _lib.selftest_stream(src[(i % 4) * n:], dst[(i % 4) * (n // 2):], sink, n, mode)
-            for i in range(3):
-                launch(i)
-            evs = [torch.cuda.Event(enable_timing=True) for _ in range(21)]
-            evs[0].record()
-            for i in range(20):
-                launch(i)
-                evs[i + 1].record()
-            torch.cuda.synchronize()
-            us = sorted(evs[i].elapsed_time(evs[i + 1]) * 1e3 for i in range(20))[10]
-            res[name] = {"us_median": us, "bytes": moved, "TBps": moved / us / 1e6}
-        print(json.dumps({"stream_calibration": res}))
-        return
-
-    if args.issue_calibration:
-        torch.cuda.set_device(0)
-        cus = torch.cuda.get_device_properties(0).multi_processor_count
-        wps, reps = 3, 2000                             # wavefronts per SIMD; 4 * reps repetitions per wavefront
-        blocks = cus * wps                              # 256 threads = one wavefront per SIMD of a CU
-        out = torch.empty(blocks * 256, dtype=torch.float32, device="cuda")
-        res = {}
-        for kind, name in ((0, "v_mfma_i32_32x32x32_i8"), (1, "v_mfma_f32_32x32x64_f8f6f4"), (2, "v_mfma_f32_32x32x16_f16")):
-            row = {}
-            for nv in (0, 8, 16, 32, 64):
-                _lib.selftest_issue(out, kind, nv, reps, blocks)
-                torch.cuda.synchronize()
-                e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-                e0.record()
-                _lib.selftest_issue(out, kind, nv, reps, blocks)
-                e1.record()
-                torch.cuda.synchronize()
-                row[str(nv)] = e0.elapsed_time(e1) * 1e6 / (4.0 * reps) / wps      # ns per (MFMA + nv adds) per SIMD
-            slope = (row["64"] - row["32"]) / 32.0                                   # ns per add once the adds dominate
-            row["ns_per_add"] = slope
-            row["mfma_share_ns"] = row["32"] - 32.0 * slope      # what an MFMA adds to a stream of vector adds
-            res[name] = row
-        print(json.dumps({"issue_calibration": {"wavefronts_per_simd": wps, "unit": "ns per (one MFMA + NV v_add_f32) per SIMD",
-                                                "kinds": res}}))
         return
 
     cfg = W.CONFIGS[args.config]

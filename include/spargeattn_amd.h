@@ -7,7 +7,8 @@
  * of thu-ml/SpargeAttn.  Every function takes raw DEVICE pointers, explicit
  * sizes, enum ints and a HIP stream (hipStream_t passed as void*); it launches
  * asynchronously on that stream, allocates nothing, synchronises nothing and
- * keeps no state.  Tensors the library produces are contiguous (B,H,N,D) ("HND"); the caller's own q, k, v and output
+ * keeps no state - with one exception, spg_km_mean_static, which owns an 8 MiB
+ * device array per GPU and remembers its address (see there).  Tensors the library produces are contiguous (B,H,N,D) ("HND"); the caller's own q, k, v and output
  * may be strided (see "Strides" below).
  * Return value: SPG_OK or an error code; spg_last_error() gives the message of
  * the last failure on the calling thread.
@@ -38,6 +39,14 @@ enum spg_dtype { SPG_F16 = 0, SPG_BF16 = 1 };
  * when no row's running maximum came within pvthreshd of being raised by it - never, decided for the whole 128-row
  * Q block (the mode every Python entry point of the reference uses), or for each 32 query rows on their own. */
 enum spg_pv_threshold_mode { SPG_PV_NONE = 0, SPG_PV_PER_BLOCK = 1, SPG_PV_PER_WARP = 2 };
+
+/* qk_quant_gran of the reference's kernel entry points (csrc/qattn/attn_cuda.h:61-76, dispatched in
+ * csrc/pytorch_extensions_utils.cuh:71-85; QuantGranularity in csrc/qattn/attn_utils.cuh:44-50), same integer values:
+ * 1 = one INT8 scale per 128-row Q block and per 64-row K block (what every Python operator of the reference passes),
+ * 2 = one scale per warp: 32 query rows (q_scale (B,H,nq*4), index 4*qblock + row/32, csrc/qattn/qk_int_sv_f8_cuda_sm89.cuh:111-115)
+ *     and 64 key rows, i.e. K scales stay per block (WARP_K = CTA_K = 64);
+ * 3 = per thread: tied to the lane layout of mma.sync fragments, refused with SPG_ERR_UNSUPPORTED. */
+enum spg_qk_quant_gran { SPG_QUANT_PER_BLOCK = 1, SPG_QUANT_PER_WARP = 2 };
 
 /* element kinds accepted for a user block mask ("non-zero = keep", spas_sage_attn/utils.py:68-69) */
 enum spg_mask_kind {
@@ -79,10 +88,15 @@ int spg_km_mean_static(const void *k, const int64_t *k_strides, void *km, int B,
  * replaces triton_bmm_pool_sim_simmean_fuse_quant (spas_sage_attn/utils.py:161-214, wrapper 270-280).
  * x (B,H,N,D) dtype, strided; km (B,H,D) dtype or NULL (Q: NULL, K: the column mean, subtracted in dtype);
  * block = 128 (Q) or 64 (K); simthreshd1 (H,) float32.
- * out: pool (B,H,nb,D) dtype; sim (B,H,nb) uint8 0/1; xq (B,H,N,D) int8; scale (B,H,nb) float32.
+ * quant_rows = rows that share one INT8 scale: `block` for per-block scales (the reference's operators), or 32 with
+ * block = 128 and km == NULL for the per-warp granularity of Q (per_warp_int8 with WARPQ = 32,
+ * spas_sage_attn/quant_per_block.py:102-148, same arithmetic as the fused kernel): nb * block / quant_rows scales per
+ * head, a 32-row group without rows (past N in the last block) gets the scale of an all-zero group, 1e-7.
+ * out: pool (B,H,nb,D) dtype; sim (B,H,nb) uint8 0/1; xq (B,H,N,D) int8; scale (B,H,nb*block/quant_rows) float32.
  * ---- A13: with pool == NULL and sim == NULL this is qk_quantize (utils.py:89-159): xq and scale only. */
 int spg_pool_sim_quant(const void *x, const int64_t *x_strides, const void *km, void *pool, uint8_t *sim, int8_t *xq,
-                       float *scale, const float *simthreshd1, int B, int H, int N, int D, int block, int dtype, void *stream);
+                       float *scale, const float *simthreshd1, int B, int H, int N, int D, int block, int quant_rows,
+                       int dtype, void *stream);
 
 /* ---- A5-A8: compressed attention, top-k / CDF selection, block map, LUT ------------------------
  * replaces the torch glue of get_block_map_meansim_fuse_quant (spas_sage_attn/utils.py:386-420),
@@ -117,12 +131,14 @@ int spg_v_quant_fp8(const void *v, const int64_t *v_strides, uint8_t *v8, float 
 /* ---- A11: block-sparse INT8-QK / FP8-PV attention ------------------------------------------------
  * replaces qk_int8_sv_f8_accum_f32_block_sparse_attn_inst_buf_fuse_v_scale_with_pv_threshold
  * (csrc/qattn/attn_cuda.h:61-76, csrc/qattn/qk_int_sv_f8_cuda_sm89.cu:197-390) with
- * tensor_layout = HND, qk_quant_gran = per-block; pv_threshold_mode = SPG_PV_PER_BLOCK is what that entry point
- * compiles in (sm89.cu:365), the other two modes are the kernel template's (sm89.cuh:283-391).
+ * tensor_layout = HND; qk_quant_gran as that entry point takes it (1 per block, 2 per warp; 3 is refused);
+ * pv_threshold_mode = SPG_PV_PER_BLOCK is what that entry point compiles in (sm89.cu:365), the other two modes are the
+ * kernel template's (sm89.cuh:283-391).
  * q8 int8 (B,H,N,D); k8 int8 (B,Hkv,N_kv,D); v8 as produced by spg_v_quant_fp8 for Hkv heads of N_kv rows; out (B,H,N,D)
  * out_dtype, strided.  N (qo_len) and N_kv (kv_len) are independent as in the reference (sm89.cu:256-300):
  * nq = ceil(N/128), nk = ceil(N_kv/64); keys >= N_kv of the last block are masked.
- * lut (B,H,nq,nk) / valid_block_num as above; pvthreshd (H,) float32; q_scale (B,H,nq), k_scale (B,Hkv,nk),
+ * lut (B,H,nq,nk) / valid_block_num as above; pvthreshd (H,) float32; q_scale (B,H,nq) for qk_quant_gran = 1 or
+ * (B,H,nq*4) for qk_quant_gran = 2, k_scale (B,Hkv,nk),
  * v_scale (B,Hkv,D) float32; Hkv divides H: query head h reads K/V head h / (H / Hkv) (grouped-query attention,
  * sm89.cu:310-314, sm89.cuh:118); Hkv = H is plain multi-head attention; pv_count (B,H,nq*4) int32 or NULL: number of K blocks
  * whose PV was computed, one entry per 32 query rows as in the reference (sm89.cu:331-334); entries of Q blocks with
@@ -132,7 +148,7 @@ int spg_block_sparse_attn(const int8_t *q8, const int8_t *k8, const uint8_t *v8,
                           int out_dtype, const int32_t *lut, const int32_t *valid_block_num, const float *pvthreshd,
                           const float *q_scale, const float *k_scale, const float *v_scale,
                           int B, int H, int Hkv, int N, int N_kv, int D, float sm_scale, int is_causal,
-                          int pv_threshold_mode, int32_t *pv_count, void *stream);
+                          int qk_quant_gran, int pv_threshold_mode, int32_t *pv_count, void *stream);
 
 /* ---- SageAttention1-style variant: INT8 QK^T, FP16 PV.
  * Replaces qk_int8_sv_f16_accum_f16_block_sparse_attn_inst_buf_with_pv_threshold (csrc/qattn/attn_cuda.h:32-45,
@@ -148,7 +164,7 @@ int spg_block_sparse_attn_f16v(const int8_t *q8, const int8_t *k8, const void *v
                                int out_dtype, const int32_t *lut, const int32_t *valid_block_num, const float *pvthreshd,
                                const float *q_scale, const float *k_scale,
                                int B, int H, int Hkv, int N, int N_kv, int D, float sm_scale, int is_causal,
-                               int pv_threshold_mode, int32_t *pv_count, void *stream);
+                               int qk_quant_gran, int pv_threshold_mode, int32_t *pv_count, void *stream);
 
 /* ---- measurement comparator: dense FP16 flash attention on MFMA (no counterpart in the reference;
  * the "dense FP16 attention kernel built in the same run" the speed-up is quoted against).
@@ -170,18 +186,6 @@ int spg_selftest_division(unsigned long long *counts, int n_divisors, unsigned i
  * cannot reach because P = 2^x with x <= 8.807);
  * saturate == 0: the bare v_cvt_pk_fp8_f32 instruction (NaN for |x| > 464), for documentation of the hardware. */
 int spg_selftest_fp8_pack(const float *x, uint8_t *codes, int n, int saturate, void *stream);
-
-/* ---- measurement aid (no counterpart in the reference): what the machine delivers for the access shapes of the
- * streaming kernels, with nothing but the loads and stores.  mode 0: read `bytes` from src, 16 B per lane, non-temporal
- * hint; mode 1: the same with plain loads; mode 2: read `bytes` (non-temporal) and write bytes/2 to dst (the 2-bytes-in,
- * 1-byte-out shape of the quantisation kernels).  bytes is a multiple of 32768; sink is 4 writable bytes. */
-int spg_selftest_stream(const void *src, void *dst, void *sink, size_t bytes, int mode, void *stream);
-
-/* ---- measurement aid (no counterpart in the reference): how matrix and vector instructions share a SIMD.  Every
- * wavefront of `blocks` workgroups (256 threads) repeats 4 * reps times "one MFMA, then nv independent v_add_f32" with two
- * accumulator chains.  kind 0: v_mfma_i32_32x32x32_i8, 1: v_mfma_f32_32x32x64_f8f6f4, 2: v_mfma_f32_32x32x16_f16;
- * nv in {0, 8, 16, 32, 64}; out: blocks * 256 floats. */
-int spg_selftest_issue(float *out, int kind, int nv, int reps, int blocks, void *stream);
 
 #ifdef __cplusplus
 }

@@ -26,7 +26,7 @@ def hyperparameter(h, value):
     return a
 
 
-def _common_tail(res, q, v, dtype, pvthreshd, scale, kernel_causal):
+def _common_tail(res, q, v, dtype, pvthreshd, scale, kernel_causal, qk_quant_gran=1):
     b, h, n, d = q.shape
     v16 = vq.to_fp16(v)
     v8, v_scale = vq.v_quant_fp8(v16)
@@ -35,15 +35,23 @@ def _common_tail(res, q, v, dtype, pvthreshd, scale, kernel_causal):
     out, written, pvc = at.block_sparse_attention(
         res["q8"], res["k8"], v8, res["lut"], res["valid"], hyperparameter(h, pvthreshd),
         res["q_scale"], res["k_scale"], v_scale, sm_scale, dtype,
-        is_causal=kernel_causal, return_pv_count=True)
+        is_causal=kernel_causal, return_pv_count=True, qk_quant_gran=qk_quant_gran)
     res["out"], res["written"], res["pv_count"] = out, written, pvc
     return res
 
 
+def _q_rows(qk_quant_gran):
+    """Rows of Q that share an INT8 scale: the 128-row block, or the 32 rows of a warp (quant_per_block.py:102-148)."""
+    assert qk_quant_gran in (1, 2)
+    return mp.BLKQ if qk_quant_gran == 1 else 32
+
+
 def spas_sage2_attn_meansim_topk(q, k, v, dtype, is_causal=False, scale=None, simthreshd1=-0.1,
                                  cdfthreshd=None, topk=0.5, pvthreshd=50, attention_sink=False,
-                                 kernel_causal=False, stop_after_mask=False):
-    """core.py:105-169.  ``kernel_causal`` is the flag the reference always passes as False (core.py:154-158)."""
+                                 kernel_causal=False, stop_after_mask=False, qk_quant_gran=1):
+    """core.py:105-169.  ``kernel_causal`` is the flag the reference always passes as False (core.py:154-158);
+    ``qk_quant_gran`` is the kernel's granularity argument, which the reference's operator fixes at 1 (core.py:156):
+    with 2, Q is quantised in 32-row groups and the kernel reads one scale per warp."""
     q = np.asarray(q, dtype=F32)
     k = np.asarray(k, dtype=F32)
     b, h, n, d = q.shape
@@ -52,7 +60,7 @@ def spas_sage2_attn_meansim_topk(q, k, v, dtype, is_causal=False, scale=None, si
     km = mp.km_mean(k, dtype)
     res["km"] = km
     thr = hyperparameter(h, simthreshd1)
-    rq = mp.pool_sim_quant(q, None, mp.BLKQ, thr, dtype)
+    rq = mp.pool_sim_quant(q, None, mp.BLKQ, thr, dtype, quant_rows=_q_rows(qk_quant_gran))
     # grouped K/V heads (not in the reference, whose pooled-score matmul needs equal head counts): K is pooled once per
     # K head with the similarity threshold of the first query head of its group
     rk = mp.pool_sim_quant(k, km, mp.BLKK, thr[::h // k.shape[1]], dtype)
@@ -72,16 +80,16 @@ def spas_sage2_attn_meansim_topk(q, k, v, dtype, is_causal=False, scale=None, si
         res["sparsity"] = 1 - tot / ((nk + 2) // 2 * nq * b * h)       # core.py:166
     if stop_after_mask:
         return res
-    return _common_tail(res, q, v, dtype, pvthreshd, scale, kernel_causal)
+    return _common_tail(res, q, v, dtype, pvthreshd, scale, kernel_causal, qk_quant_gran)
 
 
 def spas_sage_attn_meansim_topk(q, k, v, dtype, is_causal=False, scale=None, simthreshd1=-0.1, cdfthreshd=None,
-                                topk=0.5, pvthreshd=50, attention_sink=False):
+                                topk=0.5, pvthreshd=50, attention_sink=False, qk_quant_gran=1):
     """core.py:278-319 (and 235-276 with cdfthreshd): the mask prediction of the Sage2 operator, then the INT8-QK /
     FP16-PV kernel on fp16(v) with the token-level causal flag (core.py:308-310)."""
     res = spas_sage2_attn_meansim_topk(q, k, v, dtype, is_causal=is_causal, scale=scale, simthreshd1=simthreshd1,
                                        cdfthreshd=cdfthreshd, topk=topk, attention_sink=attention_sink,
-                                       stop_after_mask=True)
+                                       stop_after_mask=True, qk_quant_gran=qk_quant_gran)
     q = np.asarray(q, dtype=F32)
     b, h, n, d = q.shape
     hkv, nkv = np.shape(v)[1], np.shape(v)[2]              # K/V may have fewer heads and another length than Q
@@ -92,12 +100,13 @@ def spas_sage_attn_meansim_topk(q, k, v, dtype, is_causal=False, scale=None, sim
     sm_scale = (1.0 / d ** 0.5) if scale is None else scale
     out, written, pvc = at.block_sparse_attention(
         res["q8"], res["k8"], v16, res["lut"], res["valid"], hyperparameter(h, pvthreshd), res["q_scale"],
-        res["k_scale"], None, sm_scale, dtype, is_causal=bool(is_causal), return_pv_count=True, pv="f16")
+        res["k_scale"], None, sm_scale, dtype, is_causal=bool(is_causal), return_pv_count=True, pv="f16",
+        qk_quant_gran=qk_quant_gran)
     res["out"], res["written"], res["pv_count"] = out, written, pvc
     return res
 
 
-def block_sparse_sage2_attn(q, k, v, mask_id, dtype, scale=None, pvthreshd=50, kernel_causal=False):
+def block_sparse_sage2_attn(q, k, v, mask_id, dtype, scale=None, pvthreshd=50, kernel_causal=False, qk_quant_gran=1):
     """core.py:171-233 (get_vanilla_qk_quant + block_map_lut_triton + kernel)."""
     q = np.asarray(q, dtype=F32)
     k = np.asarray(k, dtype=F32)
@@ -106,10 +115,10 @@ def block_sparse_sage2_attn(q, k, v, mask_id, dtype, scale=None, pvthreshd=50, k
     res = {}
     km = mp.km_mean(k, dtype)
     res["km"] = km
-    rq = mp.pool_sim_quant(q, None, mp.BLKQ, None, dtype, with_pool=False)
+    rq = mp.pool_sim_quant(q, None, mp.BLKQ, None, dtype, with_pool=False, quant_rows=_q_rows(qk_quant_gran))
     rk = mp.pool_sim_quant(k, km, mp.BLKK, None, dtype, with_pool=False)
     res.update(q8=rq["q"], q_scale=rq["scale"], k8=rk["q"], k_scale=rk["scale"])
     res["lut"], res["valid"] = mp.map_to_lut(mask_id)
     nq, nk = res["lut"].shape[2], res["lut"].shape[3]
     res["sparsity"] = 1 - float(res["valid"].astype(F32).sum()) / ((nk + 2) // 2 * nq * b * h)  # core.py:230
-    return _common_tail(res, q, v, dtype, pvthreshd, scale, kernel_causal)
+    return _common_tail(res, q, v, dtype, pvthreshd, scale, kernel_causal, qk_quant_gran)

@@ -47,7 +47,8 @@ def _fma(a, b, c):
 
 
 def block_sparse_attention(q8, k8, v8, lut, valid, pvthreshd, q_scale, k_scale, v_scale,
-                           sm_scale, out_dtype, is_causal=False, return_pv_count=False, pv="fp8", pv_mode=1):
+                           sm_scale, out_dtype, is_causal=False, return_pv_count=False, pv="fp8", pv_mode=1,
+                           qk_quant_gran=1):
     """q8,k8 int8 (B,H,N,D); v8 e4m3 codes uint8 (B,H,Npad,D); lut/valid int32.
 
     Returns (out float32 (B,H,N,D) holding out_dtype values, written (B,H,nq) bool[, pv_count (B,H,nq)]).
@@ -55,6 +56,10 @@ def block_sparse_attention(q8, k8, v8, lut, valid, pvthreshd, q_scale, k_scale, 
     ``pv_mode`` is the kernel template's PVThresholdMode (attn_utils.cuh:58-62): 1 = the skip is decided for the whole
     128-row block (what every Python entry point uses), 2 = for each warp of 32 rows on its own (sm89.cuh:302-318
     without the block reduction of 320-343; pv_count is then (B,H,nq,4)), 0 = never skip.
+
+    ``qk_quant_gran`` is the kernel entry's granularity switch (csrc/qattn/attn_cuda.h:61-76): 1 = q_scale (B,H,nq), one
+    scale per 128-row block; 2 = q_scale (B,H,nq*4), one per warp of 32 query rows, read at 4*block + row//32
+    (sm89.cuh:111-115).  K scales are (B,Hkv,nk) in both (a K "warp" spans the whole 64-row block, sm89.cuh:123-131).
 
     ``pv="f16"`` restates the SageAttention1 kernel instead (qk_int_sv_f16_cuda_sm80.cuh:42-671 instantiated with
     per-block quantisation, per-block PV threshold and the row sum on the tensor cores, sm80.cuh:690): ``v8`` then holds
@@ -65,7 +70,7 @@ def block_sparse_attention(q8, k8, v8, lut, valid, pvthreshd, q_scale, k_scale, 
     the block to its binary32 accumulator (compute_fp16_sv_permuted_inst_buf, attn_utils.cuh:683-751) - parity
     unpinned for that rounding, the comparison is by tolerance.
     """
-    assert pv in ("fp8", "f16") and pv_mode in (0, 1, 2)
+    assert pv in ("fp8", "f16") and pv_mode in (0, 1, 2) and qk_quant_gran in (1, 2)
     q8 = np.asarray(q8)
     k8 = np.asarray(k8)
     b_, h_, n, d_ = q8.shape
@@ -96,7 +101,10 @@ def block_sparse_attention(q8, k8, v8, lut, valid, pvthreshd, q_scale, k_scale, 
                 dsum = np.ones(CTA_Q, dtype=F32)
                 o = np.zeros((CTA_Q, d_), dtype=F32)
                 idxs = np.cumsum(lut[b, h, i, :nv].astype(np.int64))
-                qs = F32(q_scale[b, h, i])
+                if qk_quant_gran == 1:
+                    qs = np.full(CTA_Q, q_scale[b, h, i], dtype=F32)
+                else:
+                    qs = np.repeat(np.asarray(q_scale[b, h, 4 * i:4 * i + 4], dtype=F32), 32)
                 cnt = np.zeros(4, dtype=np.int32)
                 for it, j in enumerate(idxs):
                     c0 = int(j) * CTA_K
@@ -105,10 +113,10 @@ def block_sparse_attention(q8, k8, v8, lut, valid, pvthreshd, q_scale, k_scale, 
                     kb[:cols] = k8[b, hk, c0:c0 + cols]
                     vb = vf[b, hk, c0:c0 + CTA_K]
                     s = (qb @ kb.T).astype(F32)                 # exact integers
-                    dq = F32(qs * F32(k_scale[b, hk, j]))
+                    dq = (qs * F32(k_scale[b, hk, j])).astype(F32)[:, None]      # per query row
                     if it < nv - 2:
-                        a = F32(c * dq)
-                        m_blk = (s.max(axis=1) * a).astype(F32)
+                        a = (c * dq).astype(F32)
+                        m_blk = (s.max(axis=1) * a[:, 0]).astype(F32)
                         d_row = (m_blk - m).astype(F32)
                         if pv_mode == 1:
                             act4 = np.full(4, bool(F32(np.max(d_row) + thr) > 0))

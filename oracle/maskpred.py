@@ -162,12 +162,18 @@ def quant_int8_block(xb):
     return q, scale
 
 
-def pool_sim_quant(x, km, bs, simthreshd1, dtype, with_pool=True):
+def pool_sim_quant(x, km, bs, simthreshd1, dtype, with_pool=True, quant_rows=None):
     """One pass of the fused Triton kernel over x (B,H,N,D) T-typed float32.
 
     km: (B,H,D) T-typed or None.  simthreshd1: (H,) float32.
     Returns dict(pool (B,H,nb,D) T, sim (B,H,nb) bool, q (B,H,N,D) int8, scale (B,H,nb) f32).
     With ``with_pool=False`` this is ``qk_quantize`` (utils.py:89-159): q and scale only.
+
+    ``quant_rows`` (a divisor of ``bs``; default ``bs``) is the number of rows that share one INT8 scale.  32 with
+    bs = 128 is the per-warp granularity of Q: ``per_warp_int8`` (spas_sage_attn/quant_per_block.py:102-148) launches
+    the same per-group arithmetic (quant_per_block.py:41-48 = utils.py:140-148) over nb * bs / 32 groups per head, a
+    group past the end of the tensor included (all masked -> scale 1e-7); scale is then (B,H,nb*bs/quant_rows).
+    Pooling and the similarity flag are per block of ``bs`` rows whatever the granularity.
     """
     x = np.asarray(x, dtype=F32)
     b, h, n, d = x.shape
@@ -176,7 +182,9 @@ def pool_sim_quant(x, km, bs, simthreshd1, dtype, with_pool=True):
     xb, rows_valid, valid = _blocked(x, bs)
     xb = np.where(valid[None, None, :, :, None], xb, F32(0))   # utils.py:188 (re-zero masked rows)
     nb = xb.shape[2]
-    q, scale = quant_int8_block(xb)
+    qr = bs if quant_rows is None else int(quant_rows)
+    assert qr > 0 and bs % qr == 0
+    q, scale = quant_int8_block(xb.reshape(b, h, nb * (bs // qr), qr, d))
     out = {"q": q.reshape(b, h, nb * bs, d)[:, :, :n, :], "scale": scale}
     if not with_pool:
         return out

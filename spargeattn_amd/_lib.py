@@ -10,8 +10,7 @@ import os
 import torch
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-# SPARGEATTN_AMD_LIB lets a developer point at another build of the same library (A/B comparisons)
-LIB_PATH = os.environ.get("SPARGEATTN_AMD_LIB", os.path.join(_HERE, "libspargeattn_amd.so"))
+LIB_PATH = os.path.join(_HERE, "libspargeattn_amd.so")
 
 SPG_OK, SPG_ERR_INVALID, SPG_ERR_UNSUPPORTED, SPG_ERR_HIP = 0, 1, 2, 3
 SPG_F16, SPG_BF16 = 0, 1
@@ -26,18 +25,16 @@ SIGNATURES = {
     "spg_km_mean_workspace_bytes": (_sz, [_i, _i, _i, _i]),
     "spg_km_mean": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp]),
     "spg_km_mean_static": (_i, [_vp, _vp, _vp, _i, _i, _i, _i, _i, _vp]),
-    "spg_pool_sim_quant": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp]),
+    "spg_pool_sim_quant": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _vp]),
     "spg_block_select": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _vp]),
     "spg_map_to_lut": (_i, [_vp, _i, _vp, _vp, _i, _i, _i, _i, _vp]),
     "spg_v_quant_fp8": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp]),
-    "spg_block_sparse_attn": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _f, _i, _i, _vp, _vp]),
+    "spg_block_sparse_attn": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _f, _i, _i, _i, _vp, _vp]),
     "spg_v_tiles_f16": (_i, [_vp, _vp, _vp, _i, _i, _i, _i, _i, _vp]),
-    "spg_block_sparse_attn_f16v": (_i, [_vp] * 5 + [_i] + [_vp] * 5 + [_i] * 6 + [_f, _i, _i, _vp, _vp]),
+    "spg_block_sparse_attn_f16v": (_i, [_vp] * 5 + [_i] + [_vp] * 5 + [_i] * 6 + [_f, _i, _i, _i, _vp, _vp]),
     "spg_dense_attn_f16": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _f, _i, _vp]),
     "spg_selftest_division": (_i, [_vp, _i, ctypes.c_uint, _vp]),
     "spg_selftest_fp8_pack": (_i, [_vp, _vp, _i, _i, _vp]),
-    "spg_selftest_stream": (_i, [_vp, _vp, _vp, ctypes.c_size_t, _i, _vp]),
-    "spg_selftest_issue": (_i, [_vp, _i, _i, _i, _i, _vp]),
 }
 
 _lib = None
@@ -140,20 +137,25 @@ def km_mean(k):
     return km
 
 
-def pool_sim_quant(x, km, block, simthreshd1=None, with_pool=True, stream=None):
-    """Returns (pool, sim, x_int8, scale) - pool and sim are None when with_pool is False."""
+def pool_sim_quant(x, km, block, simthreshd1=None, with_pool=True, stream=None, quant_rows=None):
+    """Returns (pool, sim, x_int8, scale) - pool and sim are None when with_pool is False.
+    quant_rows: rows that share one INT8 scale (default: the block; 32 for the per-warp granularity of Q), scale is
+    (B, H, nb * block / quant_rows)."""
     _dev_strided(x)
     _dev(km, simthreshd1)
     B, H, N, D = x.shape
     nb = (N + block - 1) // block
+    quant_rows = block if quant_rows is None else int(quant_rows)
+    if quant_rows <= 0 or block % quant_rows:
+        raise ValueError(f"quant_rows ({quant_rows}) must divide the block size ({block})")
     xq = torch.empty((B, H, N, D), dtype=torch.int8, device=x.device)
-    scale = torch.empty((B, H, nb), dtype=torch.float32, device=x.device)
+    scale = torch.empty((B, H, nb * (block // quant_rows)), dtype=torch.float32, device=x.device)
     pool = sim = None
     if with_pool:
         pool = torch.empty((B, H, nb, D), dtype=x.dtype, device=x.device)
         sim = torch.empty((B, H, nb), dtype=torch.bool, device=x.device)
     _check(load().spg_pool_sim_quant(_p(x), _st(x), _p(km), _p(pool), _p(sim), _p(xq), _p(scale), _p(simthreshd1),
-                                     B, H, N, D, block, _dt(x), _stream(stream)))
+                                     B, H, N, D, block, quant_rows, _dt(x), _stream(stream)))
     return pool, sim, xq, scale
 
 
@@ -225,9 +227,22 @@ def v8_natural_to_tiles(v8_nat):
 
 
 PV_NONE, PV_PER_BLOCK, PV_PER_WARP = 0, 1, 2
+QUANT_PER_BLOCK, QUANT_PER_WARP = 1, 2
 
 
-def _check_attn_shapes(q8, k8, vt, lut, valid, q_scale, k_scale, v_scale=None):
+def quant_gran(value):
+    """qk_quant_gran as the reference's kernel entry takes it (1 per block, 2 per warp, 3 per thread,
+    csrc/pytorch_extensions_utils.cuh:71-85) or by name -> 1 or 2; anything else raises ValueError."""
+    names = {"per_block": 1, "per_warp": 2, "per_thread": 3}
+    g = names.get(value, value) if isinstance(value, str) else value
+    if g in (QUANT_PER_BLOCK, QUANT_PER_WARP) and not isinstance(g, bool):
+        return int(g)
+    if g == 3:
+        raise ValueError("qk_quant_gran 3 (per thread) is not supported on gfx950")
+    raise ValueError(f"Unsupported qk_quant_gran: {value}")
+
+
+def _check_attn_shapes(q8, k8, vt, lut, valid, q_scale, k_scale, v_scale=None, qk_quant_gran=QUANT_PER_BLOCK):
     """Shapes the attention kernels index with: raises before a launch could read past a buffer.
     The query length N and the key/value length N_kv are independent (qo_len / kv_len of
     csrc/qattn/qk_int_sv_f8_cuda_sm89.cu:256-300)."""
@@ -241,25 +256,27 @@ def _check_attn_shapes(q8, k8, vt, lut, valid, q_scale, k_scale, v_scale=None):
     if tuple(lut.shape) != (B, H, nq, nk) or tuple(valid.shape) != (B, H, nq):
         raise RuntimeError(f"lut / valid_block_num have shapes {tuple(lut.shape)} / {tuple(valid.shape)}, "
                            f"expected {(B, H, nq, nk)} / {(B, H, nq)}")
-    if tuple(q_scale.shape) != (B, H, nq) or tuple(k_scale.shape) != (B, Hkv, nk):
+    nqs = nq * 4 if qk_quant_gran == QUANT_PER_WARP else nq
+    if tuple(q_scale.shape) != (B, H, nqs) or tuple(k_scale.shape) != (B, Hkv, nk):
         raise RuntimeError(f"q_scale / k_scale have shapes {tuple(q_scale.shape)} / {tuple(k_scale.shape)}, "
-                           f"expected {(B, H, nq)} / {(B, Hkv, nk)}")
+                           f"expected {(B, H, nqs)} / {(B, Hkv, nk)} for qk_quant_gran = {qk_quant_gran}")
     if v_scale is not None and tuple(v_scale.shape) != (B, Hkv, D):
         raise RuntimeError(f"v_scale has shape {tuple(v_scale.shape)}, expected {(B, Hkv, D)}")
     return B, H, Hkv, N, Nk, D
 
 
 def block_sparse_attn(q8, k8, v8, out, lut, valid, pvthreshd, q_scale, k_scale, v_scale, sm_scale,
-                      is_causal=False, return_pv_count=False, pv_mode=PV_PER_BLOCK):
+                      is_causal=False, return_pv_count=False, pv_mode=PV_PER_BLOCK, qk_quant_gran=QUANT_PER_BLOCK):
     _dev(q8, k8, v8, lut, valid, pvthreshd, q_scale, k_scale, v_scale)
     _dev_strided(out)
-    B, H, Hkv, N, Nk, D = _check_attn_shapes(q8, k8, v8, lut, valid, q_scale, k_scale, v_scale)
+    qk_quant_gran = quant_gran(qk_quant_gran)
+    B, H, Hkv, N, Nk, D = _check_attn_shapes(q8, k8, v8, lut, valid, q_scale, k_scale, v_scale, qk_quant_gran)
     if tuple(out.shape) != (B, H, N, D) or pvthreshd.numel() != H:
         raise RuntimeError("out must have q's shape and pvthreshd one entry per query head")
     pvc = torch.zeros((B, H, 4 * ((N + 127) // 128)), dtype=torch.int32, device=q8.device) if return_pv_count else None
     _check(load().spg_block_sparse_attn(_p(q8), _p(k8), _p(v8), _p(out), _st(out), _dt(out), _p(lut), _p(valid), _p(pvthreshd),
                                         _p(q_scale), _p(k_scale), _p(v_scale), B, H, Hkv, N, Nk, D, float(sm_scale),
-                                        int(bool(is_causal)), int(pv_mode), _p(pvc), _stream()))
+                                        int(bool(is_causal)), qk_quant_gran, int(pv_mode), _p(pvc), _stream()))
     return pvc
 
 
@@ -284,16 +301,17 @@ def v_tiles_f16_to_natural(vt):
 
 
 def block_sparse_attn_f16v(q8, k8, vt, out, lut, valid, pvthreshd, q_scale, k_scale, sm_scale, is_causal=False,
-                           return_pv_count=False, pv_mode=PV_PER_BLOCK):
+                           return_pv_count=False, pv_mode=PV_PER_BLOCK, qk_quant_gran=QUANT_PER_BLOCK):
     _dev(q8, k8, vt, lut, valid, pvthreshd, q_scale, k_scale)
     _dev_strided(out)
-    B, H, Hkv, N, Nk, D = _check_attn_shapes(q8, k8, vt, lut, valid, q_scale, k_scale)
+    qk_quant_gran = quant_gran(qk_quant_gran)
+    B, H, Hkv, N, Nk, D = _check_attn_shapes(q8, k8, vt, lut, valid, q_scale, k_scale, None, qk_quant_gran)
     if tuple(out.shape) != (B, H, N, D) or pvthreshd.numel() != H:
         raise RuntimeError("out must have q's shape and pvthreshd one entry per query head")
     pvc = torch.zeros((B, H, 4 * ((N + 127) // 128)), dtype=torch.int32, device=q8.device) if return_pv_count else None
     _check(load().spg_block_sparse_attn_f16v(_p(q8), _p(k8), _p(vt), _p(out), _st(out), _dt(out), _p(lut), _p(valid),
                                              _p(pvthreshd), _p(q_scale), _p(k_scale), B, H, Hkv, N, Nk, D, float(sm_scale),
-                                             int(bool(is_causal)), int(pv_mode), _p(pvc), _stream()))
+                                             int(bool(is_causal)), qk_quant_gran, int(pv_mode), _p(pvc), _stream()))
     return pvc
 
 
@@ -316,21 +334,6 @@ def selftest_fp8_pack(x, saturate=True):
     codes = torch.empty(x.numel(), dtype=torch.uint8, device=x.device)
     _check(load().spg_selftest_fp8_pack(_p(x), _p(codes), x.numel(), int(bool(saturate)), _stream()))
     return codes.view(x.shape)
-
-
-def selftest_stream(src, dst, sink, nbytes, mode):
-    """Launches the streaming probe once: mode 0 / 1 read nbytes of src (non-temporal / plain loads), mode 2 reads nbytes
-    and writes nbytes / 2 to dst."""
-    _dev(src, sink)
-    _check(load().spg_selftest_stream(_p(src), _p(dst) if dst is not None else None, _p(sink), int(nbytes), int(mode),
-                                      _stream()))
-
-
-def selftest_issue(out, kind, nv, reps, blocks):
-    """Launches the issue probe once: every wavefront repeats 4 * reps times one MFMA of `kind` + nv vector adds."""
-    _dev(out)
-    assert out.dtype == torch.float32 and out.numel() >= blocks * 256
-    _check(load().spg_selftest_issue(_p(out), int(kind), int(nv), int(reps), int(blocks), _stream()))
 
 
 def selftest_division(n_divisors, seed=1):

@@ -25,7 +25,6 @@ SOURCES = {
     "vquant.hip": ["-ffp-contract=off"],
     "attn.hip": [],
     "dense.hip": [],
-    "probe.hip": [],
     "capi.hip": ["-fvisibility=default"],
 }
 # Translation units whose kernels read LDS through inline asm into registers the compiler believes are already

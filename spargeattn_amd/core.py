@@ -12,6 +12,9 @@ callers need no change; everything runs as HIP kernels for gfx950.  As in the re
 fp16 for fp32/fp16 inputs and bf16 for bf16 inputs, and causality is enforced at 128x64-block
 granularity through the LUT (the reference passes ``is_causal=False`` to its kernel, core.py:154-158).
 ``kernel_causal=True`` is an extension that additionally masks at token level.
+``qk_quant_gran`` (keyword, default 1 = the reference's operators) selects the INT8 granularity of the kernel entry
+(csrc/qattn/attn_cuda.h:61-76): 1 / "per_block", or 2 / "per_warp" - one Q scale per 32 query rows
+(spas_sage_attn/quant_per_block.py:102-148), which lowers the quantisation error at no cost in time.
 """
 import torch
 
@@ -81,7 +84,7 @@ def _empty_out(q):
 
 
 def _attention(q, k, v, q_int8, q_scale, k_int8, k_scale, lut, valid_block_num, scale, pvthreshd, kernel_causal,
-               return_pv_count=False):
+               return_pv_count=False, qk_quant_gran=1):
     headdim = q.size(-1)
     if scale is None:
         scale = 1.0 / (headdim ** 0.5)
@@ -92,7 +95,8 @@ def _attention(q, k, v, q_int8, q_scale, k_int8, k_scale, lut, valid_block_num, 
     v_fp8, v_scale = _lib.v_quant_fp8(v)
     _mark("attn")
     pvc = _lib.block_sparse_attn(q_int8, k_int8, v_fp8, o, lut, valid_block_num, pvthreshd, q_scale, k_scale, v_scale,
-                                 scale, is_causal=kernel_causal, return_pv_count=return_pv_count)
+                                 scale, is_causal=kernel_causal, return_pv_count=return_pv_count,
+                                 qk_quant_gran=qk_quant_gran)
     _mark("end")
     return o, pvc
 
@@ -109,7 +113,8 @@ def _finish(o, tensor_layout, return_sparsity, valid_block_num, lut, causal_deno
 
 
 def _meansim(q, k, v, is_causal, scale, smooth_k, simthreshd1, cdfthreshd, topk, pvthreshd, attention_sink,
-             tensor_layout, return_sparsity, kernel_causal):
+             tensor_layout, return_sparsity, kernel_causal, qk_quant_gran=1):
+    qk_quant_gran = _lib.quant_gran(qk_quant_gran)
     q, k, v = _prologue(q, k, v, tensor_layout)
     if not smooth_k:
         # the reference leaves `km` undefined in this case (core.py:119-126)
@@ -119,15 +124,17 @@ def _meansim(q, k, v, is_causal, scale, smooth_k, simthreshd1, cdfthreshd, topk,
     _mark("maskpred")
     lut, valid_block_num, q_int8, q_scale, k_int8, k_scale = get_block_map_meansim_fuse_quant(
         q, k, km, is_causal=is_causal, simthreshd1=simthreshd1, cdfthreshd=cdfthreshd, topk=topk, return_lut=True,
-        attention_sink=attention_sink, BLKQ=128, BLKK=64)
-    o, _ = _attention(q, k, v, q_int8, q_scale, k_int8, k_scale, lut, valid_block_num, scale, pvthreshd, kernel_causal)
+        attention_sink=attention_sink, BLKQ=128, BLKK=64, qk_quant_gran=qk_quant_gran)
+    o, _ = _attention(q, k, v, q_int8, q_scale, k_int8, k_scale, lut, valid_block_num, scale, pvthreshd, kernel_causal,
+                      qk_quant_gran=qk_quant_gran)
     return _finish(o, tensor_layout, return_sparsity, valid_block_num, lut, causal_denominator=is_causal is not False)
 
 
 def _meansim_sage1(q, k, v, is_causal, scale, smooth_k, simthreshd1, cdfthreshd, topk, pvthreshd, attention_sink,
-                   tensor_layout, return_sparsity):
+                   tensor_layout, return_sparsity, qk_quant_gran=1):
     """INT8 QK^T / FP16 PV path (spas_sage_attn/core.py:235-319): fp16 V, token-level causal masking in the kernel,
     sparsity reported against the full grid unless is_causal."""
+    qk_quant_gran = _lib.quant_gran(qk_quant_gran)
     q, k, v = _prologue(q, k, v, tensor_layout)
     if not smooth_k:
         raise NameError("name 'km' is not defined")           # as the reference (core.py:249-252)
@@ -136,7 +143,7 @@ def _meansim_sage1(q, k, v, is_causal, scale, smooth_k, simthreshd1, cdfthreshd,
     _mark("maskpred")
     lut, valid_block_num, q_int8, q_scale, k_int8, k_scale = get_block_map_meansim_fuse_quant(
         q, k, km, is_causal=is_causal, simthreshd1=simthreshd1, cdfthreshd=cdfthreshd, topk=topk, return_lut=True,
-        attention_sink=attention_sink)
+        attention_sink=attention_sink, qk_quant_gran=qk_quant_gran)
     headdim = q.size(-1)
     if scale is None:
         scale = 1.0 / (headdim ** 0.5)
@@ -147,7 +154,7 @@ def _meansim_sage1(q, k, v, is_causal, scale, smooth_k, simthreshd1, cdfthreshd,
     vt = _lib.v_tiles_f16_swizzled(v)
     _mark("attn")
     _lib.block_sparse_attn_f16v(q_int8, k_int8, vt, o, lut, valid_block_num, pvthreshd, q_scale, k_scale, scale,
-                                is_causal=bool(is_causal))
+                                is_causal=bool(is_causal), qk_quant_gran=qk_quant_gran)
     _mark("end")
     return _finish(o, tensor_layout, return_sparsity, valid_block_num, lut, causal_denominator=is_causal is not False)
 
@@ -155,50 +162,53 @@ def _meansim_sage1(q, k, v, is_causal, scale, smooth_k, simthreshd1, cdfthreshd,
 @torch.compiler.disable
 def spas_sage_attn_meansim_cuda(q, k, v, attn_mask=None, dropout_p=0.0, is_causal=False, scale=None, smooth_k=True,
                                 simthreshd1=0.6, cdfthreshd=0.98, pvthreshd=50, attention_sink=False,
-                                tensor_layout="HND", output_dtype=torch.float16, return_sparsity=False):
+                                tensor_layout="HND", output_dtype=torch.float16, return_sparsity=False, *,
+                                qk_quant_gran=1):
     return _meansim_sage1(q, k, v, is_causal, scale, smooth_k, simthreshd1, cdfthreshd, None, pvthreshd,
-                          attention_sink, tensor_layout, return_sparsity)
+                          attention_sink, tensor_layout, return_sparsity, qk_quant_gran)
 
 
 @torch.compiler.disable
 def spas_sage_attn_meansim_topk_cuda(q, k, v, attn_mask=None, dropout_p=0.0, is_causal=False, scale=None,
                                      smooth_k=True, simthreshd1=-0.1, cdfthreshd=None, topk=0.5, pvthreshd=50,
                                      attention_sink=False, tensor_layout="HND", output_dtype=torch.float16,
-                                     return_sparsity=False):
+                                     return_sparsity=False, *, qk_quant_gran=1):
     return _meansim_sage1(q, k, v, is_causal, scale, smooth_k, simthreshd1, cdfthreshd, topk, pvthreshd,
-                          attention_sink, tensor_layout, return_sparsity)
+                          attention_sink, tensor_layout, return_sparsity, qk_quant_gran)
 
 
 @torch.compiler.disable
 def spas_sage2_attn_meansim_cuda(q, k, v, attn_mask=None, dropout_p=0.0, is_causal=False, scale=None, smooth_k=True,
                                  simthreshd1=0.6, cdfthreshd=0.98, pvthreshd=50, attention_sink=False,
                                  tensor_layout="HND", output_dtype=torch.float16, return_sparsity=False,
-                                 kernel_causal=False):
+                                 kernel_causal=False, *, qk_quant_gran=1):
     return _meansim(q, k, v, is_causal, scale, smooth_k, simthreshd1, cdfthreshd, None, pvthreshd, attention_sink,
-                    tensor_layout, return_sparsity, kernel_causal)
+                    tensor_layout, return_sparsity, kernel_causal, qk_quant_gran)
 
 
 @torch.compiler.disable
 def spas_sage2_attn_meansim_topk_cuda(q, k, v, attn_mask=None, dropout_p=0.0, is_causal=False, scale=None,
                                       smooth_k=True, simthreshd1=-0.1, cdfthreshd=None, topk=0.5, pvthreshd=50,
                                       attention_sink=False, tensor_layout="HND", output_dtype=torch.float16,
-                                      return_sparsity=False, kernel_causal=False):
+                                      return_sparsity=False, kernel_causal=False, *, qk_quant_gran=1):
     return _meansim(q, k, v, is_causal, scale, smooth_k, simthreshd1, cdfthreshd, topk, pvthreshd, attention_sink,
-                    tensor_layout, return_sparsity, kernel_causal)
+                    tensor_layout, return_sparsity, kernel_causal, qk_quant_gran)
 
 
 @torch.compiler.disable
 def block_sparse_sage2_attn_cuda(q, k, v, mask_id=None, dropout_p=0.0, scale=None, smooth_k=True, pvthreshd=50,
                                  attention_sink=False, tensor_layout="HND", output_dtype=torch.float16,
-                                 return_sparsity=False, kernel_causal=False):
+                                 return_sparsity=False, kernel_causal=False, *, qk_quant_gran=1):
+    qk_quant_gran = _lib.quant_gran(qk_quant_gran)
     q, k, v = _prologue(q, k, v, tensor_layout)
     if not smooth_k:
         raise NameError("name 'km' is not defined")
     _mark("km")
     km = _lib.km_mean(k)
     _mark("maskpred")
-    q_int8, q_scale, k_int8, k_scale = get_vanilla_qk_quant(q, k, km, 128, 64)
+    q_int8, q_scale, k_int8, k_scale = get_vanilla_qk_quant(q, k, km, 128, 64, qk_quant_gran=qk_quant_gran)
     lut, valid_block_num = block_map_lut_triton(block_map=mask_id)
-    o, _ = _attention(q, k, v, q_int8, q_scale, k_int8, k_scale, lut, valid_block_num, scale, pvthreshd, kernel_causal)
+    o, _ = _attention(q, k, v, q_int8, q_scale, k_int8, k_scale, lut, valid_block_num, scale, pvthreshd, kernel_causal,
+                      qk_quant_gran=qk_quant_gran)
     # the reference always reports against the causal denominator here (core.py:230)
     return _finish(o, tensor_layout, return_sparsity, valid_block_num, lut, causal_denominator=True)

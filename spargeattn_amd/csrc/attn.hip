@@ -2,8 +2,8 @@
 //
 // Replaces qk_int_sv_f8_block_sparse_attn_kernel (csrc/qattn/qk_int_sv_f8_cuda_sm89.cuh:42-755) as launched by
 // qk_int8_sv_f8_accum_f32_block_sparse_attn_inst_buf_fuse_v_scale_with_pv_threshold
-// (csrc/qattn/qk_int_sv_f8_cuda_sm89.cu:197-390): per-block INT8 scales, per-block PV threshold, fp32 PV
-// accumulation, V scale fused into the epilogue.
+// (csrc/qattn/qk_int_sv_f8_cuda_sm89.cu:197-390): per-block or per-warp INT8 scales (qk_quant_gran 1 / 2), PV threshold
+// per block (or per 32 rows, or none), fp32 PV accumulation, V scale fused into the epilogue.
 //
 // Design (not a translation of the mma.sync tiling):
 //  * one workgroup = one 128-row Q block = 4 wavefronts x 32 queries;
@@ -58,6 +58,7 @@ struct AttnParams {
   float sm_scale_log2;
   int is_causal;
   int pv_mode;     // PVThresholdMode of the reference (attn_utils.cuh:58-62): 0 none, 1 per block, 2 per wavefront of 32 rows
+  int q_per_warp;  // QuantGranularity of Q (sm89.cuh:106-121): 0 one scale per 128-row block, 1 one per 32 rows (B,H,nq*4)
   int total_wg, wg_per_xcd;
 };
 
@@ -185,7 +186,9 @@ __global__ __launch_bounds__(256, PV16 ? 2 : 3) void block_sparse_attn_kernel(co
   typedef const __attribute__((address_space(4))) float *c_f32_t;
   const c_i32_t lutc = (c_i32_t)(p.lut + ((size_t)bh * p.nq + qb) * p.nk);
   const c_f32_t kscale = (c_f32_t)(p.k_scale + (size_t)bhk * p.nk);
-  const float qs = ((c_f32_t)p.q_scale)[(size_t)bh * p.nq + qb];
+  // per-warp granularity: the 32 query rows of a wavefront are one quantisation group, so the scale stays a scalar
+  const size_t qsi = (size_t)bh * p.nq + qb;
+  const float qs = ((c_f32_t)p.q_scale)[p.q_per_warp ? qsi * 4 + wave : qsi];
   const float c = p.sm_scale_log2;
   const float thr = ((c_f32_t)p.pvthr)[head];
 
@@ -358,7 +361,7 @@ __global__ __launch_bounds__(256, PV16 ? 2 : 3) void block_sparse_attn_kernel(co
     // The constant 1/(2 pi) leaves the exponent through ONE additive term, -(1/(2 pi) a 2^26 + m) (+ 8.807), whose rounding
     // error is half an ulp of 1.07e7 a.  Below 2^14 that is at most 2^-11 in the exponent (3e-4 relative in P, and the
     // row maximum's P stays below 448.2).  At or above it (large |q| |k| or a large softmax scale; uniform for the
-    // workgroup) the scores are first taken relative to the lane's own maximum - an exact subtraction inside one binade -
+    // wavefront) the scores are first taken relative to the lane's own maximum - an exact subtraction inside one binade -
     // so that no large constant is left to round: one more instruction per score, on such blocks only.
     const bool precise = __builtin_bit_cast(int, ksc) >= kscale_precise_bits;
     float fm, mloc = acc_c;
@@ -608,8 +611,8 @@ __global__ __launch_bounds__(256, PV16 ? 2 : 3) void block_sparse_attn_kernel(co
 hipError_t launch_block_sparse_attn(const int8_t *q8, const int8_t *k8, const uint8_t *v8, void *out, Strides os,
                                     int out_dtype, const int32_t *lut, const int32_t *valid, const float *pvthreshd,
                                     const float *q_scale, const float *k_scale, const float *v_scale, int B, int H,
-                                    int Hkv, int N, int Nk, int D, float sm_scale, int is_causal, int pv_mode,
-                                    int32_t *pv_count, hipStream_t st) {
+                                    int Hkv, int N, int Nk, int D, float sm_scale, int is_causal, int q_per_warp,
+                                    int pv_mode, int32_t *pv_count, hipStream_t st) {
   AttnParams p;
   p.q8 = q8; p.k8 = k8; p.v8 = v8; p.out = out; p.os = os; p.lut = lut; p.valid = valid; p.pvthr = pvthreshd;
   p.q_scale = q_scale; p.k_scale = k_scale; p.v_scale = v_scale; p.pv_count = pv_count;
@@ -617,6 +620,7 @@ hipError_t launch_block_sparse_attn(const int8_t *q8, const int8_t *k8, const ui
   p.sm_scale_log2 = sm_scale * SPG_LOG2E;
   p.is_causal = is_causal;
   p.pv_mode = pv_mode;
+  p.q_per_warp = q_per_warp;
   p.total_wg = p.nq * H * B;
   p.wg_per_xcd = (p.total_wg + 7) / 8;
   const int grid = p.wg_per_xcd * 8;

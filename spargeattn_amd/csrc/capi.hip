@@ -1,5 +1,6 @@
 // extern "C" entry points declared in include/spargeattn_amd.h: argument checks, then a launch on the caller's
-// stream.  No allocation, no synchronisation, no global state (the error string is thread-local).
+// stream.  No allocation, no synchronisation; the only state is the thread-local error string and, behind
+// spg_km_mean_static, a library-owned device array per GPU with its cached address.
 #include "../../include/spargeattn_amd.h"
 #include "launch.h"
 
@@ -42,6 +43,14 @@ int check_pv_mode(const char *fn, int mode) {
   if (mode < SPG_PV_NONE || mode > SPG_PV_PER_WARP)
     return fail(SPG_ERR_INVALID, "%s: pv_threshold_mode must be 0 (none), 1 (per block) or 2 (per 32 query rows), got %d", fn, mode);
   return SPG_OK;
+}
+
+// qk_quant_gran of the reference's kernel entry (csrc/pytorch_extensions_utils.cuh:71-85): 1 per block, 2 per warp,
+// 3 per thread.  Per-thread scales follow the lane layout of mma.sync fragments and have no counterpart here.
+int check_quant_gran(const char *fn, int gran) {
+  if (gran == SPG_QUANT_PER_BLOCK || gran == SPG_QUANT_PER_WARP) return SPG_OK;
+  if (gran == 3) return fail(SPG_ERR_UNSUPPORTED, "%s: qk_quant_gran 3 (per thread) is not supported on gfx950", fn);
+  return fail(SPG_ERR_INVALID, "%s: Unsupported qk_quant_gran: %d", fn, gran);
 }
 
 int check_dtype(const char *fn, int dtype) {
@@ -105,17 +114,22 @@ int spg_km_mean_static(const void *k, const int64_t *k_strides, void *km, int B,
 }
 
 int spg_pool_sim_quant(const void *x, const int64_t *x_strides, const void *km, void *pool, uint8_t *sim, int8_t *xq, float *scale,
-                       const float *simthreshd1, int B, int H, int N, int D, int block, int dtype, void *stream) {
+                       const float *simthreshd1, int B, int H, int N, int D, int block, int quant_rows, int dtype, void *stream) {
   const char *fn = "spg_pool_sim_quant";
   SPG_TRY(check_shape(fn, B, H, N, D));
   SPG_TRY(check_dtype(fn, dtype));
   if (block != 64 && block != 128) return fail(SPG_ERR_UNSUPPORTED, "%s: block must be 64 or 128 (got %d)", fn, block);
+  if (quant_rows != block && !(quant_rows == 32 && block == 128 && km == nullptr))
+    return fail(SPG_ERR_UNSUPPORTED, "%s: quant_rows must equal block (per-block scales), or be 32 with block = 128 and no "
+                "mean (per-warp scales of Q); got quant_rows = %d, block = %d, km %s", fn, quant_rows, block,
+                km == nullptr ? "NULL" : "given");
   SPG_NONNULL(fn, x); SPG_NONNULL(fn, xq); SPG_NONNULL(fn, scale);
   if ((pool == nullptr) != (sim == nullptr)) return fail(SPG_ERR_INVALID, "%s: pool and sim must both be given or both be NULL", fn);
   if (pool != nullptr) SPG_NONNULL(fn, simthreshd1);
   spg::Strides xs;
   SPG_TRY(get_strides(fn, "x_strides", x_strides, H, N, D, &xs));
-  spg::launch_pool_sim_quant(x, xs, km, pool, sim, xq, scale, simthreshd1, B, H, N, D, block, dtype, (hipStream_t)stream);
+  spg::launch_pool_sim_quant(x, xs, km, pool, sim, xq, scale, simthreshd1, B, H, N, D, block, quant_rows, dtype,
+                             (hipStream_t)stream);
   return check_launch(fn, hipSuccess);
 }
 
@@ -165,26 +179,6 @@ int spg_selftest_fp8_pack(const float *x, uint8_t *codes, int n, int saturate, v
   return check_launch(fn, hipSuccess);
 }
 
-int spg_selftest_stream(const void *src, void *dst, void *sink, size_t bytes, int mode, void *stream) {
-  const char *fn = "spg_selftest_stream";
-  if (bytes == 0 || bytes % 32768 != 0 || bytes / 32768 > 0x7fffffffull)
-    return fail(SPG_ERR_INVALID, "%s: bytes must be a positive multiple of 32768 (got %zu)", fn, bytes);
-  if (mode < 0 || mode > 2) return fail(SPG_ERR_INVALID, "%s: mode must be 0, 1 or 2 (got %d)", fn, mode);
-  SPG_NONNULL(fn, src); SPG_NONNULL(fn, sink);
-  if (mode == 2) SPG_NONNULL(fn, dst);
-  spg::launch_stream_probe(src, dst, sink, bytes, mode, (hipStream_t)stream);
-  return check_launch(fn, hipSuccess);
-}
-
-int spg_selftest_issue(float *out, int kind, int nv, int reps, int blocks, void *stream) {
-  const char *fn = "spg_selftest_issue";
-  if (reps <= 0 || blocks <= 0) return fail(SPG_ERR_INVALID, "%s: reps and blocks must be positive", fn);
-  SPG_NONNULL(fn, out);
-  if (!spg::launch_issue_probe(out, kind, nv, reps, blocks, (hipStream_t)stream))
-    return fail(SPG_ERR_INVALID, "%s: kind must be 0, 1 or 2 and nv one of 0, 8, 16, 32, 64 (got %d, %d)", fn, kind, nv);
-  return check_launch(fn, hipSuccess);
-}
-
 int spg_v_quant_fp8(const void *v, const int64_t *v_strides, uint8_t *v8, float *v_scale, int B, int H, int N, int D, int dtype, void *stream) {
   const char *fn = "spg_v_quant_fp8";
   SPG_TRY(check_shape(fn, B, H, N, D));
@@ -200,11 +194,13 @@ int spg_block_sparse_attn(const int8_t *q8, const int8_t *k8, const uint8_t *v8,
                           int out_dtype,
                           const int32_t *lut, const int32_t *valid_block_num, const float *pvthreshd,
                           const float *q_scale, const float *k_scale, const float *v_scale, int B, int H, int Hkv, int N,
-                          int N_kv, int D, float sm_scale, int is_causal, int pv_threshold_mode, int32_t *pv_count, void *stream) {
+                          int N_kv, int D, float sm_scale, int is_causal, int qk_quant_gran, int pv_threshold_mode,
+                          int32_t *pv_count, void *stream) {
   const char *fn = "spg_block_sparse_attn";
   SPG_TRY(check_shape(fn, B, H, N, D));
   SPG_TRY(check_shape(fn, B, Hkv > 0 ? Hkv : 1, N_kv, D));
   SPG_TRY(check_kv_heads(fn, H, Hkv));
+  SPG_TRY(check_quant_gran(fn, qk_quant_gran));
   SPG_TRY(check_pv_mode(fn, pv_threshold_mode));
   SPG_TRY(check_dtype(fn, out_dtype));
   SPG_NONNULL(fn, q8); SPG_NONNULL(fn, k8); SPG_NONNULL(fn, v8); SPG_NONNULL(fn, out); SPG_NONNULL(fn, lut);
@@ -214,7 +210,8 @@ int spg_block_sparse_attn(const int8_t *q8, const int8_t *k8, const uint8_t *v8,
   SPG_TRY(get_strides(fn, "out_strides", out_strides, H, N, D, &os));
   return check_launch(fn, spg::launch_block_sparse_attn(q8, k8, v8, out, os, out_dtype, lut, valid_block_num, pvthreshd,
                                                         q_scale, k_scale, v_scale, B, H, Hkv, N, N_kv, D, sm_scale,
-                                                        is_causal ? 1 : 0, pv_threshold_mode, pv_count, (hipStream_t)stream));
+                                                        is_causal ? 1 : 0, qk_quant_gran == SPG_QUANT_PER_WARP ? 1 : 0,
+                                                        pv_threshold_mode, pv_count, (hipStream_t)stream));
 }
 
 int spg_v_tiles_f16(const void *v, const int64_t *v_strides, void *vt, int B, int H, int N, int D, int dtype, void *stream) {
@@ -232,11 +229,13 @@ int spg_block_sparse_attn_f16v(const int8_t *q8, const int8_t *k8, const void *v
                                int out_dtype,
                                const int32_t *lut, const int32_t *valid_block_num, const float *pvthreshd,
                                const float *q_scale, const float *k_scale, int B, int H, int Hkv, int N, int N_kv, int D,
-                               float sm_scale, int is_causal, int pv_threshold_mode, int32_t *pv_count, void *stream) {
+                               float sm_scale, int is_causal, int qk_quant_gran, int pv_threshold_mode, int32_t *pv_count,
+                               void *stream) {
   const char *fn = "spg_block_sparse_attn_f16v";
   SPG_TRY(check_shape(fn, B, H, N, D));
   SPG_TRY(check_shape(fn, B, Hkv > 0 ? Hkv : 1, N_kv, D));
   SPG_TRY(check_kv_heads(fn, H, Hkv));
+  SPG_TRY(check_quant_gran(fn, qk_quant_gran));
   SPG_TRY(check_pv_mode(fn, pv_threshold_mode));
   SPG_TRY(check_dtype(fn, out_dtype));
   SPG_NONNULL(fn, q8); SPG_NONNULL(fn, k8); SPG_NONNULL(fn, vt); SPG_NONNULL(fn, out); SPG_NONNULL(fn, lut);
@@ -245,7 +244,8 @@ int spg_block_sparse_attn_f16v(const int8_t *q8, const int8_t *k8, const void *v
   SPG_TRY(get_strides(fn, "out_strides", out_strides, H, N, D, &os));
   return check_launch(fn, spg::launch_block_sparse_attn(q8, k8, (const uint8_t *)vt, out, os, out_dtype, lut, valid_block_num,
                                                         pvthreshd, q_scale, k_scale, nullptr, B, H, Hkv, N, N_kv, D, sm_scale,
-                                                        is_causal ? 1 : 0, pv_threshold_mode, pv_count, (hipStream_t)stream));
+                                                        is_causal ? 1 : 0, qk_quant_gran == SPG_QUANT_PER_WARP ? 1 : 0,
+                                                        pv_threshold_mode, pv_count, (hipStream_t)stream));
 }
 
 int spg_dense_attn_f16(const void *q, const void *k, const void *v, void *out, int B, int H, int N, int D,

@@ -20,7 +20,8 @@ void launch_km_mean(const void *k, Strides ks, void *km, void *ws, int B, int H,
 size_t km_mean_static_capacity();
 hipError_t launch_km_mean_static(const void *k, Strides ks, void *km, int B, int H, int N, int D, int dtype, hipStream_t st);
 void launch_pool_sim_quant(const void *x, Strides xs, const void *km, void *pool, uint8_t *sim, int8_t *xq, float *scale,
-                           const float *thr, int B, int H, int N, int D, int block, int dtype, hipStream_t st);
+                           const float *thr, int B, int H, int N, int D, int block, int quant_rows, int dtype,
+                           hipStream_t st);
 int block_select_max_nk();
 hipError_t launch_block_select(const void *pq, const uint8_t *sq, const void *pk, const uint8_t *sk, const float *topk,
                                const float *cdf, int causal, int sink, int32_t *lut, int32_t *valid, uint8_t *bmap,
@@ -38,11 +39,9 @@ hipError_t launch_block_sparse_attn(const int8_t *q8, const int8_t *k8, const ui
                                     int out_dtype,
                                     const int32_t *lut, const int32_t *valid, const float *pvthreshd,
                                     const float *q_scale, const float *k_scale, const float *v_scale, int B, int H,
-                                    int Hkv, int N, int Nk, int D, float sm_scale, int is_causal, int pv_mode,
-                                    int32_t *pv_count, hipStream_t st);
+                                    int Hkv, int N, int Nk, int D, float sm_scale, int is_causal, int q_per_warp,
+                                    int pv_mode, int32_t *pv_count, hipStream_t st);
 void launch_fp8_pack_selftest(const float *x, uint8_t *codes, int n, int saturate, hipStream_t st);
-void launch_stream_probe(const void *src, void *dst, void *sink, size_t bytes, int mode, hipStream_t st);
-bool launch_issue_probe(float *out, int kind, int nv, int reps, int blocks, hipStream_t st);
 
 hipError_t launch_dense_attn_f16(const void *q, const void *k, const void *v, void *out, int B, int H, int N, int D,
                                  float sm_scale, int is_causal, hipStream_t st);

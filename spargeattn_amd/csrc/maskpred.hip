@@ -189,7 +189,10 @@ __device__ __forceinline__ uint32_t wave_max_u32(uint32_t v) {
 
 // One workgroup handles 128 consecutive rows of one (batch, head): one 128-row block or two 64-row blocks (SUB), so
 // that the per-block tail (column reduction, pooled mean, flag, scale) is spread over all four wavefronts in both cases.
-template <int BS, int D, int DT, bool HAS_MEAN, bool WITH_POOL>
+// QR = rows that share one INT8 scale: BS (per-block granularity, what the reference's operators use) or 32 rows of a
+// 128-row Q block (per-warp granularity: quant_per_block.py:102-148 with WARPQ = 32, one scale per 32 query rows, which
+// are the rows of one wavefront of the attention kernel).  Pooling and the similarity flag stay per block.
+template <int BS, int D, int DT, bool HAS_MEAN, bool WITH_POOL, int QR = BS>
 __global__ __launch_bounds__(256) void pool_sim_quant_kernel(const uint16_t *__restrict__ x, const Strides xs,
                                                              const uint16_t *__restrict__ km,
                                                              uint16_t *__restrict__ pool, uint8_t *__restrict__ sim,
@@ -202,7 +205,12 @@ __global__ __launch_bounds__(256) void pool_sim_quant_kernel(const uint16_t *__r
   constexpr int NPT = ROWS / RPP;     // passes (rows per thread)
   constexpr int NP = BS / RPP;        // passes per block
   constexpr int WPS = D / 64;         // wavefronts that hold one block's columns in the tail (thread = block * D + column)
+  constexpr int NQG = ROWS / QR;      // quantisation groups per workgroup (1, 2 or 4)
+  constexpr int GPB = BS / QR;        // ... per block
+  constexpr int NPQ = QR / RPP;       // passes per quantisation group
   static_assert(BS == 64 || BS == 128, "block sizes of the operators");
+  static_assert(QR == BS || (QR == 32 && BS == 128), "per-block, or 32-row groups of a Q block");
+  static_assert(RPP <= QR, "a pass of the workgroup stays inside one quantisation group");
   static_assert(RPP <= BS && SUB * D <= 256, "thread <-> (block, column) mapping of the tail");
   // magnitude patterns (sign bit cleared) order like the magnitudes, for both 16-bit formats
   constexpr uint32_t ABS2 = 0x7fff7fffu;
@@ -256,27 +264,38 @@ __global__ __launch_bounds__(256) void pool_sim_quant_kernel(const uint16_t *__r
       if (r + p * RPP >= rows_here) { w[p][0] = 0; w[p][1] = 0; w[p][2] = 0; w[p][3] = 0; }
   }
 
-  // largest magnitude of the thread's elements per block (as 16-bit patterns: block 0 in the low half, block 1 in the
-  // high half) and, per row, whether all of the thread's elements are tiny
-  uint32_t m_thread = 0, tiny_rows = 0;
+  // largest magnitude of the thread's elements per quantisation group (as 16-bit patterns: group g in half g % 2 of
+  // word g / 2) and, per row, whether all of the thread's elements are tiny
+  constexpr int MW = (NQG + 1) / 2;
+  uint32_t m_thread[MW], tiny_rows = 0;
 #pragma unroll
-  for (int sb = 0; sb < SUB; sb++) {
+  for (int i = 0; i < MW; i++) m_thread[i] = 0;
+#pragma unroll
+  for (int g = 0; g < NQG; g++) {
     uint32_t m2 = 0;
 #pragma unroll
-    for (int p = sb * NP; p < (sb + 1) * NP; p++) {
+    for (int p = g * NPQ; p < (g + 1) * NPQ; p++) {
       const uint32_t rm = pk_max_u16(pk_max_u16(w[p][0] & ABS2, w[p][1] & ABS2), pk_max_u16(w[p][2] & ABS2, w[p][3] & ABS2));
       m2 = pk_max_u16(m2, rm);
       if constexpr (WITH_POOL) tiny_rows |= ((rm & TINY2) == 0 ? 1u : 0u) << p;
     }
-    m_thread |= max(m2 & 0xffffu, m2 >> 16) << (16 * sb);
+    m_thread[g / 2] |= max(m2 & 0xffffu, m2 >> 16) << (16 * (g % 2));
   }
-  __shared__ uint32_t s_wmax[4], s_wbad[4];
+  // largest magnitude pattern of block sb as this thread (or, after the reduction, the workgroup) knows it
+  auto block_max = [&](const uint32_t(&mm)[MW], int sb) -> uint32_t {
+    uint32_t m = 0;
+#pragma unroll
+    for (int g = sb * GPB; g < (sb + 1) * GPB; g++) m = max(m, (mm[g / 2] >> (16 * (g % 2))) & 0xffffu);
+    return m;
+  };
+  __shared__ uint32_t s_wmax[4][MW], s_wbad[4];
   __shared__ long long s_wg[4];
-  {
-    uint32_t mw = m_thread;                       // both blocks' maxima reduced together
+#pragma unroll
+  for (int i = 0; i < MW; i++) {
+    uint32_t mw = m_thread[i];                    // two groups' maxima reduced together
 #pragma unroll
     for (int o = 32; o >= 1; o >>= 1) mw = pk_max_u16(mw, (uint32_t)__shfl_xor((int)mw, o, SPG_WAVE));
-    if ((tid & 63) == 0) s_wmax[tid >> 6] = mw;
+    if ((tid & 63) == 0) s_wmax[tid >> 6][i] = mw;
   }
 
   if constexpr (WITH_POOL) {
@@ -322,7 +341,7 @@ __global__ __launch_bounds__(256) void pool_sim_quant_kernel(const uint16_t *__r
     if (sim_trivial) {
 #pragma unroll
       for (int sb = 0; sb < SUB; sb++)                 // inf or NaN anywhere (overflowing squares of finite values are harmless: x / inf = 0)
-        bad |= (((m_thread >> (16 * sb)) & 0xffffu) >= INF16 ? 1u : 0u) << sb;
+        bad |= (block_max(m_thread, sb) >= INF16 ? 1u : 0u) << sb;
       tiny_rows = group_and_u32<TPR>(tiny_rows);      // rows tiny in every lane of their group
       need_norms = __any(tiny_rows != 0);             // rare
     }
@@ -428,16 +447,21 @@ __global__ __launch_bounds__(256) void pool_sim_quant_kernel(const uint16_t *__r
     __syncthreads();
   }
 
-  const uint32_t m_all = pk_max_u16(pk_max_u16(s_wmax[0], s_wmax[1]), pk_max_u16(s_wmax[2], s_wmax[3]));
+  uint32_t m_all[MW];
+#pragma unroll
+  for (int i = 0; i < MW; i++)
+    m_all[i] = pk_max_u16(pk_max_u16(s_wmax[0][i], s_wmax[1][i]), pk_max_u16(s_wmax[2][i], s_wmax[3][i]));
   int8_t *qb = xq + ((size_t)bh * N + row_base) * D + c * 8;
 #pragma unroll
-  for (int sb = 0; sb < SUB; sb++) {
-    if (rows_valid_of(sb) <= 0) break;                  // workgroup-uniform
-    const float amax = elem_to_f32<DT>((uint16_t)(m_all >> (16 * sb)));
+  for (int g = 0; g < NQG; g++) {
+    // per-block scales exist for blocks with at least one row; the 32-row groups of the last Q block all get a scale
+    // (1e-7 for a group without rows, what the reference's quantiser writes for an all-masked group)
+    if (QR == BS && rows_here - g * QR <= 0) break;     // workgroup-uniform
+    const float amax = elem_to_f32<DT>((uint16_t)(m_all[g / 2] >> (16 * (g % 2))));
     const float s = amax / 127.0f + 1e-7f;
     auto quantise = [&](auto divide, auto check_rows) {
 #pragma unroll
-      for (int p = sb * NP; p < (sb + 1) * NP; p++) {
+      for (int p = g * NPQ; p < (g + 1) * NPQ; p++) {
         const int row = r + p * RPP;
         if (!decltype(check_rows)::value || row < rows_here) {
           float y[8];
@@ -468,7 +492,7 @@ __global__ __launch_bounds__(256) void pool_sim_quant_kernel(const uint16_t *__r
     } else {
       quantise([&](float v) { return v / s; }, std::true_type{});
     }
-    if (tid == 0) scale[(size_t)bh * nb + blk0 + sb] = s;
+    if (tid == 0) scale[((size_t)bh * nb + blk0) * GPB + g] = s;
   }
 }
 
@@ -1135,11 +1159,18 @@ hipError_t launch_km_mean_static(const void *k, Strides ks, void *km, int B, int
 
 template <int BS, int D, int DT>
 static void launch_psq3(const void *x, Strides xs, const void *km, void *pool, uint8_t *sim, int8_t *xq, float *scale,
-                        const float *thr, int B, int H, int N, hipStream_t st) {
+                        const float *thr, int B, int H, int N, int quant_rows, hipStream_t st) {
   const int nb = (N + BS - 1) / BS;
   const dim3 grid((N + 127) / 128, B * H);      // one workgroup per 128 rows: one or two blocks
   const uint16_t *xp = (const uint16_t *)x, *kp = (const uint16_t *)km;
   uint16_t *pp = (uint16_t *)pool;
+  if constexpr (BS == 128) {
+    if (quant_rows == 32) {                     // per-warp granularity of Q (no mean: the C ABI refuses the combination)
+      if (pool != nullptr) pool_sim_quant_kernel<BS, D, DT, false, true, 32><<<grid, 256, 0, st>>>(xp, xs, kp, pp, sim, xq, scale, thr, H, N, nb);
+      else                 pool_sim_quant_kernel<BS, D, DT, false, false, 32><<<grid, 256, 0, st>>>(xp, xs, kp, pp, sim, xq, scale, thr, H, N, nb);
+      return;
+    }
+  }
   if (pool != nullptr) {
     if (km) pool_sim_quant_kernel<BS, D, DT, true, true><<<grid, 256, 0, st>>>(xp, xs, kp, pp, sim, xq, scale, thr, H, N, nb);
     else    pool_sim_quant_kernel<BS, D, DT, false, true><<<grid, 256, 0, st>>>(xp, xs, kp, pp, sim, xq, scale, thr, H, N, nb);
@@ -1150,8 +1181,9 @@ static void launch_psq3(const void *x, Strides xs, const void *km, void *pool, u
 }
 
 void launch_pool_sim_quant(const void *x, Strides xs, const void *km, void *pool, uint8_t *sim, int8_t *xq, float *scale,
-                           const float *thr, int B, int H, int N, int D, int block, int dtype, hipStream_t st) {
-#define SPG_PSQ(BS_, D_, DT_) launch_psq3<BS_, D_, DT_>(x, xs, km, pool, sim, xq, scale, thr, B, H, N, st)
+                           const float *thr, int B, int H, int N, int D, int block, int quant_rows, int dtype,
+                           hipStream_t st) {
+#define SPG_PSQ(BS_, D_, DT_) launch_psq3<BS_, D_, DT_>(x, xs, km, pool, sim, xq, scale, thr, B, H, N, quant_rows, st)
   if (block == 128) {
     if (D == 64) { if (dtype == 0) SPG_PSQ(128, 64, 0); else SPG_PSQ(128, 64, 1); }
     else         { if (dtype == 0) SPG_PSQ(128, 128, 0); else SPG_PSQ(128, 128, 1); }

@@ -35,10 +35,17 @@ def _check_blocks(BLKQ_, BLKK_):
         raise ValueError("the gfx950 kernels use 128-row Q blocks and 64-row K blocks")
 
 
-def get_vanilla_qk_quant(q, k, km=None, BLKQ=128, BLKK=64):
-    """Per-block INT8 quantisation of q and (k - km) without pooling."""
+def _q_quant_rows(qk_quant_gran):
+    """Rows of Q that share one INT8 scale: the block, or the 32 rows of a warp / wavefront (per_warp_int8 with
+    WARPQ = 32, spas_sage_attn/quant_per_block.py:102-148).  K scales are per 64-row block in both granularities."""
+    return BLKQ if _lib.quant_gran(qk_quant_gran) == _lib.QUANT_PER_BLOCK else 32
+
+
+def get_vanilla_qk_quant(q, k, km=None, BLKQ=128, BLKK=64, qk_quant_gran=1):
+    """INT8 quantisation of q and (k - km) without pooling: per block, or with qk_quant_gran = 2 ("per_warp") one scale
+    per 32 query rows, q_scale (B,H,nq*4)."""
     _check_blocks(BLKQ, BLKK)
-    _, _, q_int8, q_scale = _lib.pool_sim_quant(q, None, BLKQ, with_pool=False)
+    _, _, q_int8, q_scale = _lib.pool_sim_quant(q, None, BLKQ, with_pool=False, quant_rows=_q_quant_rows(qk_quant_gran))
     _, _, k_int8, k_scale = _lib.pool_sim_quant(k, km, BLKK, with_pool=False)
     return q_int8, q_scale, k_int8, k_scale
 
@@ -85,8 +92,9 @@ block_map_lut = block_map_lut_triton
 
 def get_block_map_meansim_fuse_quant(q, k, km=None, is_causal=False, BLKQ=128, BLKK=64, simthreshd1=0.1,
                                      cdfthreshd=0.9, topk=None, is_sparse=True, return_lut=False,
-                                     attention_sink=False):
-    """Mask prediction fused with Q/K quantisation.
+                                     attention_sink=False, qk_quant_gran=1):
+    """Mask prediction fused with Q/K quantisation.  ``qk_quant_gran`` = 2 ("per_warp") quantises Q in 32-row groups
+    (q_scale (B,H,nq*4)); pooling, flags and the block map do not depend on it.
 
     Returns (lut, valid_block_num, q_int8, q_scale, k_int8, k_scale) when ``return_lut`` else
     (block_map bool, q_int8, q_scale, k_int8, k_scale)."""
@@ -97,15 +105,23 @@ def get_block_map_meansim_fuse_quant(q, k, km=None, is_causal=False, BLKQ=128, B
     if Hkv <= 0 or H % Hkv != 0:
         # the message of the reference's kernel entry (qk_int_sv_f8_cuda_sm89.cu:310-314)
         raise ValueError(f"num_qo_heads ({H}) must be divisible by num_kv_heads ({Hkv})")
+    per_head_sim = isinstance(simthreshd1, Tensor) and simthreshd1.dim() == 1
     simthreshd1 = hyperparameter_check(simthreshd1, H, q.device)
     if cdfthreshd is not None:
         cdfthreshd = hyperparameter_check(cdfthreshd, H, q.device)
     if topk is not None:
         topk = hyperparameter_check(topk, H, q.device)
-    pool_q, sim_q, q_int8, q_scale = _lib.pool_sim_quant(q, None, BLKQ, simthreshd1)
+    pool_q, sim_q, q_int8, q_scale = _lib.pool_sim_quant(q, None, BLKQ, simthreshd1, quant_rows=_q_quant_rows(qk_quant_gran))
     # Grouped K/V heads (an extension: the reference's pooled-score matmul needs Hkv == H, utils.py:388).  K is pooled and
-    # quantised once per K head; its similarity flags use the threshold of the FIRST query head of the group; every query
-    # head of the group is scored against those pooled blocks with its own topk / cdfthreshd.
+    # quantised once per K head, so its similarity flags can follow ONE threshold per group: the query heads of a group
+    # must agree on simthreshd1 (a per-head tensor that differs inside a group is refused rather than silently reduced
+    # to its first entry); every query head of the group is scored against those pooled blocks with its own topk /
+    # cdfthreshd.
+    if Hkv != H and per_head_sim:
+        grouped = simthreshd1.view(Hkv, H // Hkv)
+        if not bool((grouped == grouped[:, :1]).all()):
+            raise ValueError("simthreshd1 must be equal for the query heads that share a K/V head "
+                             f"({H} query heads, {Hkv} K/V heads): K is pooled once per K/V head")
     simthreshd1_k = simthreshd1 if Hkv == H else simthreshd1[::H // Hkv].contiguous()
     pool_k, sim_k, k_int8, k_scale = _lib.pool_sim_quant(k, km, BLKK, simthreshd1_k)
     lut, valid, bmap = _lib.block_select(pool_q, sim_q, pool_k, sim_k, topk=topk, cdfthreshd=cdfthreshd,

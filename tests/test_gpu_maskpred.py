@@ -246,35 +246,3 @@ def test_helper_wrappers_of_the_reference_utils():
     assert torch.equal(p2, want[0]) and torch.equal(s2, want[1])
     with pytest.raises(ValueError):
         utils.get_quant(x, None, 32)
-
-
-def test_stream_probe_copies_what_it_reads():
-    """The streaming probe (a measurement aid) really moves the bytes it is credited with: mode 2 writes, for every 16
-    bytes read, the two xor-folded words; modes 0 and 1 only read."""
-    n = 4 * 32768
-    g = torch.Generator().manual_seed(5)
-    src = torch.randint(0, 2 ** 31 - 1, (n // 4,), generator=g, dtype=torch.int32).cuda()
-    dst = torch.zeros(n // 8, dtype=torch.int32, device="cuda")
-    sink = torch.zeros(1, dtype=torch.int32, device="cuda")
-    for mode in (0, 1):
-        _lib.selftest_stream(src, None, sink, n, mode)
-    _lib.selftest_stream(src, dst, sink, n, 2)
-    w = src.view(-1, 4)
-    want = torch.stack([w[:, 0] ^ w[:, 1], w[:, 2] ^ w[:, 3]], dim=1).reshape(-1)
-    assert torch.equal(dst, want)
-    with pytest.raises(ValueError):
-        _lib.selftest_stream(src, dst, sink, 1000, 2)
-
-
-def test_issue_probe_runs_and_rejects_unknown_shapes():
-    """The issue probe (a measurement aid) launches for every MFMA kind and add count it advertises."""
-    out = torch.full((4 * 256,), float("nan"), dtype=torch.float32, device="cuda")
-    for kind in (0, 1, 2):
-        for nv in (0, 8, 16, 32, 64):
-            _lib.selftest_issue(out, kind, nv, 3, 4)
-    torch.cuda.synchronize()
-    assert torch.isfinite(out).all()
-    with pytest.raises(ValueError):
-        _lib.selftest_issue(out, 3, 8, 3, 4)
-    with pytest.raises(ValueError):
-        _lib.selftest_issue(out, 0, 7, 3, 4)
