@@ -254,11 +254,13 @@ def num_to_select_topk(topk, nk):
 def num_to_select_cdf(p, order, cdfthreshd, dtype):
     """cumsum of the sorted probabilities rounded to T, then searchsorted(right=True) (utils.py:398-403).
 
-    PARITY UNPINNED: cdf[i] is defined here as the EXACT running sum rounded once to T.  The reference calls
-    torch.cumsum on a bf16/fp16 CUDA tensor, whose scan may combine partial sums in the tensor dtype (a rounding per
-    combine step, in an order the library chooses); no fixture of the reference covers it.  On long bf16 rows such a
-    scan can stall below 1 and then counts MORE blocks for the same threshold, so a cdfthreshd tuned with the CUDA
-    reference may select a different number of blocks here.
+    cdf[i] is the EXACT running sum rounded once to T, compared with the binary32 threshold.  Pinned by
+    tests/test_oracle_cdf_pin.py against the routines the reference calls (torch.sort -> torch.cumsum ->
+    torch.searchsorted(right=True)) on CPU tensors of dtype T: torch's CPU scan accumulates in binary32 and rounds every
+    prefix once, and the counts agree on random rows, long flat rows and thresholds on / beside cdf values.
+    What stays open is the CUDA scan of the same call: if it combines partial sums in T (a rounding per combine step),
+    a long flat bf16 row stalls below 1 and counts MORE blocks for the same threshold, so a cdfthreshd tuned with the
+    CUDA reference may select fewer blocks here.
 
     p (B,H,nq,nk); cdfthreshd (H,) float32.  Returns int64 (B,H,nq).
     """
