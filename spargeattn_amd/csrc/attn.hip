@@ -222,10 +222,11 @@ __global__ __launch_bounds__(256, PV16 ? 2 : 3) void block_sparse_attn_kernel(co
     unsigned char *lk_ = sKr + (BUFOFF) + WL * wave * 1024;                                                   \
     unsigned char *lv_ = sVr + (PV16 ? 2 * (BUFOFF) : (BUFOFF)) + WLV * wave * 1024;                          \
     if ((BLK) != last_partial_blk) {                                                                          \
+      /* the loads of one tile back to back: they share the LDS base register (M0) */                          \
       __builtin_amdgcn_global_load_lds((glb_ptr_t)(kb_ + k_lane), (lds_ptr_t)lk_, 16, 0, 0);                  \
-      __builtin_amdgcn_global_load_lds((glb_ptr_t)(vb_ + v_lane), (lds_ptr_t)lv_, 16, 0, 0);                  \
       if constexpr (WL == 2)                                                                                  \
         __builtin_amdgcn_global_load_lds((glb_ptr_t)(kb_ + k_lane), (lds_ptr_t)lk_, 16, 1024, 0);             \
+      __builtin_amdgcn_global_load_lds((glb_ptr_t)(vb_ + v_lane), (lds_ptr_t)lv_, 16, 0, 0);                  \
       if constexpr (WLV >= 2)                                                                                 \
         __builtin_amdgcn_global_load_lds((glb_ptr_t)(vb_ + v_lane), (lds_ptr_t)lv_, 16, 1024, 0);             \
       if constexpr (WLV == 4) {                                                                               \
@@ -294,7 +295,8 @@ __global__ __launch_bounds__(256, PV16 ? 2 : 3) void block_sparse_attn_kernel(co
   __syncthreads();
 
   // One K block.  TAIL = false: every block but the last two - PV-threshold test, no masks (sm89.cuh:283-391).
-  // TAIL = true: the last two blocks - token-causal and out-of-bound masks, no skip (sm89.cuh:467-648).  The two are
+  // TAIL = true: the last two blocks - token-causal and out-of-bound masks where a score needs them, no skip
+  // (sm89.cuh:467-648).  The two are
   // separate loops so that the common one carries none of the tail's predicates.
   // SLOT = 0, 1, 2: the ring slot of the block is a compile-time constant (the common loop is unrolled three times), so
   // every LDS address of the iteration is a loop-invariant register plus an immediate offset; SLOT = -1: the slot is the
@@ -357,7 +359,9 @@ __global__ __launch_bounds__(256, PV16 ? 2 : 3) void block_sparse_attn_kernel(co
     __builtin_amdgcn_sched_barrier(0);
     const float dq = qs * ksc;                     // used by the tail blocks only
     // S0/S1 are never rewritten (no copies at the join of the two paths): slot e < 16 is S0[e], slot e >= 16 is S1[e - 16]
-    const float a26 = cq26 * ksc;                  // multiplier of the accumulator read as a float: a * 2^26
+    // multiplier of the accumulator read as a float: a * 2^26.  Wavefront-uniform, so it is moved to a scalar register:
+    // the 32 multiply-adds below then read two vector registers each instead of three
+    const float a26 = __builtin_bit_cast(float, __builtin_amdgcn_readfirstlane(__builtin_bit_cast(int, cq26 * ksc)));
     // The constant 1/(2 pi) leaves the exponent through ONE additive term, -(1/(2 pi) a 2^26 + m) (+ 8.807), whose rounding
     // error is half an ulp of 1.07e7 a.  Below 2^14 that is at most 2^-11 in the exponent (3e-4 relative in P, and the
     // row maximum's P stays below 448.2).  At or above it (large |q| |k| or a large softmax scale; uniform for the
@@ -366,7 +370,18 @@ __global__ __launch_bounds__(256, PV16 ? 2 : 3) void block_sparse_attn_kernel(co
     const bool precise = __builtin_bit_cast(int, ksc) >= kscale_precise_bits;
     float fm, mloc = acc_c;
     int lim = 0x7fffffff;
-    if constexpr (!TAIL) {
+    // The last two blocks take the masked arithmetic only if some score of the wavefront is masked at all (token-causal
+    // kernels near the diagonal, a partial last K block); otherwise they run the arithmetic of the common loop, which
+    // differs from the reference's masked branch (de-quantise, then scale) by the order of two binary32 roundings.
+    bool masked = false;                             // wavefront-uniform
+    if constexpr (TAIL) {
+      // slot e of this lane is key 64*blk + 32*hh + e; keys beyond `lim` are masked
+      const int key0 = blk * 64 + 32 * hh;
+      if (p.is_causal) lim = q_row - key0;                       // key > query (attn_utils.cuh:334-361)
+      if (it == nv - 1) lim = min(lim, Nk - 1 - key0);           // key >= kv_len (attn_utils.cuh:363-389)
+      masked = __any(lim < 31);
+    }
+    if (!masked) {
       int imax = S0[0];
 #pragma unroll
       for (int e = 1; e < 16; e++) imax = max(imax, S0[e]);
@@ -375,10 +390,6 @@ __global__ __launch_bounds__(256, PV16 ? 2 : 3) void block_sparse_attn_kernel(co
       mloc = __builtin_bit_cast(float, imax);   // 1/(2 pi) + 2^-26 * the largest of this lane's 32 dot products
       fm = (mloc - acc_c) * a26;                // the subtraction is exact (same binade)
     } else {
-      // slot e of this lane is key 64*blk + 32*hh + e; keys beyond `lim` are masked
-      const int key0 = blk * 64 + 32 * hh;
-      if (p.is_causal) lim = q_row - key0;                       // key > query (attn_utils.cuh:334-361)
-      if (it == nv - 1) lim = min(lim, Nk - 1 - key0);           // key >= kv_len (attn_utils.cuh:363-389)
       fm = SPG_NEG_BIG;
       const float dq26 = dq * SPG_ACC_SCALE;
 #pragma unroll
@@ -434,7 +445,7 @@ __global__ __launch_bounds__(256, PV16 ? 2 : 3) void block_sparse_attn_kernel(co
       const float neg0 = PV16 ? -m : -m + SPG_FP8_OFFSET;
       float ps;
       float x[32];
-      if constexpr (!TAIL) {
+      if (!masked) {
         // three passes kept apart for the scheduler: a multiply-add feeding the exponential of the same element directly,
         // and the exponential feeding the running sum, would issue as one long chain of dependent instructions
         if (!precise) {
