@@ -8,8 +8,9 @@
  * sizes, enum ints and a HIP stream (hipStream_t passed as void*); it launches
  * asynchronously on that stream, allocates nothing, synchronises nothing and
  * keeps no state - with one exception, spg_km_mean_static, which owns an 8 MiB
- * device array per GPU and remembers its address (see there).  Tensors the library produces are contiguous (B,H,N,D) ("HND"); the caller's own q, k, v and output
- * may be strided (see "Strides" below).
+ * device array per GPU and remembers its address (see there).  Tensors the
+ * library produces are contiguous (B,H,N,D) ("HND"); the caller's own q, k, v
+ * and output may be strided (see "Strides" below).
  * Return value: SPG_OK or an error code; spg_last_error() gives the message of
  * the last failure on the calling thread.
  *
@@ -80,7 +81,8 @@ int spg_km_mean(const void *k, const int64_t *k_strides, void *km, void *workspa
  * Limit: spg_km_mean_workspace_bytes(B,H,N,D) <= 8 MiB (any shape with B*H <= 8192 at D = 128 or B*H <= 16384 at D = 64);
  * larger shapes return SPG_ERR_UNSUPPORTED.  All calls on one GPU share the array: calls that overlap in time on one
  * GPU (two streams, two threads) race and must be ordered by the caller; calls on one stream are ordered already.
- * The first call on a device looks the array's address up (no allocation, but make it outside a graph capture). */
+ * The first call on a device looks the array's address up (no allocation, but make it outside a graph capture).
+ * `stream` must belong to the current device (SPG_ERR_INVALID otherwise): each GPU has its own copy of the array. */
 int spg_km_mean_static(const void *k, const int64_t *k_strides, void *km, int B, int H, int N, int D, int dtype,
                        void *stream);
 

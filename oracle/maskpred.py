@@ -153,12 +153,14 @@ def quant_int8_block(xb):
     Returns (int8 array, float32 scale (...)).
     """
     xb = np.asarray(xb, dtype=F32)
-    amax = np.max(np.abs(xb), axis=(-2, -1))
+    # tl.max lowers to a maxnum: NaN elements do not take part in the block maximum (an all-NaN block is not defined)
+    amax = np.fmax.reduce(np.fmax.reduce(np.abs(xb), axis=-1, initial=F32(0)), axis=-1, initial=F32(0))
     scale = (amax / F32(127.0)).astype(F32)
     scale = (scale + F32(1e-7)).astype(F32)
-    y = (xb / scale[..., None, None]).astype(F32)
-    y = (y + np.where(y >= 0, F32(0.5), F32(-0.5)).astype(F32)).astype(F32)
-    q = np.trunc(y).astype(np.int32).astype(np.int8)
+    with np.errstate(invalid="ignore"):
+        y = (xb / scale[..., None, None]).astype(F32)
+        y = (y + np.where(y >= 0, F32(0.5), F32(-0.5)).astype(F32)).astype(F32)
+        q = np.where(np.isnan(y), F32(0), np.trunc(y)).astype(np.int32).astype(np.int8)   # a NaN converts to 0
     return q, scale
 
 

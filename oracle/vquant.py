@@ -9,6 +9,7 @@ and is not restated: the oracle returns V8 in natural (B,H,Npad,D) order.
 Arithmetic (binary32, IEEE divide): amax = max_n |v16| ; v_scale = amax/2.25 ;
 recp = 2.25/amax ; V8 = e4m3_rne_satfinite(v16 * recp) ; rows N..Npad-1 are 0.
 An all-zero channel gives 0*inf = NaN codes, as in the reference (unguarded).
+NaN elements do not take part in the channel maximum (fmaxf / fminf, fused.cu:120-123) and get the NaN code.
 
 Pinned by tests/test_oracle_vquant.py: ``torch.float8_e4m3fn`` cast of the same
 product (library RNE cast), max|V8| == 2.25 per non-zero channel, dequantisation
@@ -33,7 +34,8 @@ def v_quant_fp8(v16, pad=128):
     v16 = np.asarray(v16, dtype=F32)
     b, h, n, d = v16.shape
     npad = (n + pad - 1) // pad * pad
-    amax = np.max(np.abs(v16), axis=2)
+    # fmaxf / fminf of the reference (fused.cu:120-123) ignore NaN: a NaN element poisons its own code only
+    amax = np.fmax.reduce(np.abs(v16), axis=2, initial=F32(0))
     with np.errstate(divide="ignore", invalid="ignore"):
         v_scale = (amax / SCALE_MAX).astype(F32)
         recp = (SCALE_MAX / amax).astype(F32)

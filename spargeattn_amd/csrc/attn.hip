@@ -322,9 +322,13 @@ __global__ __launch_bounds__(256, PV16 ? 2 : 3) void block_sparse_attn_kernel(co
         if constexpr (CS) lds_read_2x128<(SLOT < 0 ? 0 : SLOT) * TILE, (SLOT < 0 ? 0 : SLOT) * TILE + 16 * D>(a0[ks], a1[ks], kaddr_c[ks]);
         else lds_read_2x128<0, 16 * D>(a0[ks], a1[ks], kaddr_c[ks] + bufoff);
       };
-#pragma unroll
-      for (int ks = 0; ks < HK; ks++) read_k(ks);
-      if constexpr (HK == 2) lds_wait4(a0[0], a1[0], a0[1], a1[1]); else lds_wait2(a0[0], a1[0]);
+      // first group: nothing to overlap with, the reads carry their wait
+      {
+        constexpr int SO = CS ? SLOT * TILE : 0;
+        const uint32_t bo = CS ? 0u : bufoff;
+        if constexpr (HK == 2) lds_read_4x128_wait<SO, SO + 16 * D>(a0[0], a1[0], a0[1], a1[1], kaddr_c[0] + bo, kaddr_c[1] + bo);
+        else lds_read_2x128_wait<SO, SO + 16 * D>(a0[0], a1[0], kaddr_c[0] + bo, kaddr_c[0] + bo);
+      }
 #pragma unroll
       for (int ks = HK; ks < KS; ks++) read_k(ks);
       // the first product of each chain, with the inline constant as its C operand (the compiler would otherwise keep
@@ -510,13 +514,10 @@ __global__ __launch_bounds__(256, PV16 ? 2 : 3) void block_sparse_attn_kernel(co
         const uint32_t va = lds_v0 + 2 * bufoff + v_rd16;
         v4i t[4][NDT];
         // steps 0,1 are read first; steps 2,3 are in flight while 0,1 multiply
-#pragma unroll
-        for (int s4 = 0; s4 < 2; s4++) {
-          lds_read_2x128<0, 4096>(t[s4][0], t[s4][1], va ^ (uint32_t)(16 * s4));
-          if constexpr (NDT == 4) lds_read_2x128<8192, 12288>(t[s4][2], t[s4][3], va ^ (uint32_t)(16 * s4));
-        }
-        if constexpr (NDT == 4) { lds_wait4(t[0][0], t[0][1], t[0][2], t[0][3]); lds_wait4(t[1][0], t[1][1], t[1][2], t[1][3]); }
-        else { lds_wait4(t[0][0], t[0][1], t[1][0], t[1][1]); }
+        if constexpr (NDT == 4)
+          lds_read_8x128_wait<0, 4096, 8192, 12288>(t[0][0], t[0][1], t[0][2], t[0][3], t[1][0], t[1][1], t[1][2], t[1][3], va, va ^ 16u);
+        else
+          lds_read_4x128_wait<0, 4096>(t[0][0], t[0][1], t[1][0], t[1][1], va, va ^ 16u);
 #pragma unroll
         for (int s4 = 2; s4 < 4; s4++) {
           lds_read_2x128<0, 4096>(t[s4][0], t[s4][1], va ^ (uint32_t)(16 * s4));
@@ -545,9 +546,8 @@ __global__ __launch_bounds__(256, PV16 ? 2 : 3) void block_sparse_attn_kernel(co
         const uint32_t va_lo = CS ? va_lo_c : va_lo_c + bufoff, va_hi = CS ? va_hi_c : va_hi_c + bufoff;
         v4i lo[NDT], hi[NDT];
         // group 0 (output tile dt reads channel rows 32 dt .. 32 dt + 31: 2048 bytes further on)
-        lds_read_pair<SB>(lo[0], hi[0], va_lo, va_hi);
-        if constexpr (HD == 2) lds_read_pair<SB + 2048>(lo[1], hi[1], va_lo, va_hi);
-        if constexpr (HD == 2) lds_wait4(lo[0], hi[0], lo[1], hi[1]); else lds_wait2(lo[0], hi[0]);
+        if constexpr (HD == 2) lds_read_4x128_wait<SB, SB + 2048>(lo[0], lo[1], hi[0], hi[1], va_lo, va_hi);
+        else lds_read_2x128_wait<SB, SB>(lo[0], hi[0], va_lo, va_hi);
         // group 1 in flight while group 0 multiplies
         if constexpr (HD == 2) {
           lds_read_pair<SB + 4096>(lo[2], hi[2], va_lo, va_hi);

@@ -110,7 +110,10 @@ int spg_km_mean_static(const void *k, const int64_t *k_strides, void *km, int B,
                 "(use spg_km_mean with a workspace of your own)", fn, B, H, N, D, need, spg::km_mean_static_capacity());
   spg::Strides ks;
   SPG_TRY(get_strides(fn, "k_strides", k_strides, H, N, D, &ks));
-  return check_launch(fn, spg::launch_km_mean_static(k, ks, km, B, H, N, D, dtype, (hipStream_t)stream));
+  const hipError_t e = spg::launch_km_mean_static(k, ks, km, B, H, N, D, dtype, (hipStream_t)stream);
+  if (e == hipErrorInvalidDevice)
+    return fail(SPG_ERR_INVALID, "%s: the stream's device must be the current device (the built-in array is per GPU)", fn);
+  return check_launch(fn, e);
 }
 
 int spg_pool_sim_quant(const void *x, const int64_t *x_strides, const void *km, void *pool, uint8_t *sim, int8_t *xq, float *scale,

@@ -281,6 +281,34 @@ __global__ __launch_bounds__(256) void pool_sim_quant_kernel(const uint16_t *__r
     }
     m_thread[g / 2] |= max(m2 & 0xffffu, m2 >> 16) << (16 * (g % 2));
   }
+  // A NaN pattern lies above the infinity pattern and wins the maxima above.  The similarity flag wants exactly that
+  // (a block with a NaN is never "similar"), the quantisation scale does not: the reference's block maximum ignores NaN
+  // (tl.max lowers to a maxnum, utils.py:140 / 206), so only the NaN elements themselves are poisoned (they quantise to
+  // 0).  m_raw keeps the maxima with NaN for the flag; a thread that met one recomputes m_thread without (rare).
+  uint32_t m_raw[MW];
+#pragma unroll
+  for (int i = 0; i < MW; i++) m_raw[i] = m_thread[i];
+  {
+    bool nan_seen = false;
+#pragma unroll
+    for (int i = 0; i < MW; i++) nan_seen |= (m_thread[i] & 0xffffu) > INF16 || (m_thread[i] >> 16) > INF16;
+    if (nan_seen) {
+#pragma unroll
+      for (int i = 0; i < MW; i++) m_thread[i] = 0;
+#pragma unroll
+      for (int g = 0; g < NQG; g++) {
+        uint32_t m1 = 0;
+#pragma unroll
+        for (int p = g * NPQ; p < (g + 1) * NPQ; p++)
+#pragma unroll
+          for (int j = 0; j < 4; j++) {
+            const uint32_t lo = w[p][j] & 0x7fffu, hi = (w[p][j] >> 16) & 0x7fffu;
+            m1 = max(m1, max(lo > INF16 ? 0u : lo, hi > INF16 ? 0u : hi));
+          }
+        m_thread[g / 2] |= m1 << (16 * (g % 2));
+      }
+    }
+  }
   // largest magnitude pattern of block sb as this thread (or, after the reduction, the workgroup) knows it
   auto block_max = [&](const uint32_t(&mm)[MW], int sb) -> uint32_t {
     uint32_t m = 0;
@@ -341,7 +369,7 @@ __global__ __launch_bounds__(256) void pool_sim_quant_kernel(const uint16_t *__r
     if (sim_trivial) {
 #pragma unroll
       for (int sb = 0; sb < SUB; sb++)                 // inf or NaN anywhere (overflowing squares of finite values are harmless: x / inf = 0)
-        bad |= (block_max(m_thread, sb) >= INF16 ? 1u : 0u) << sb;
+        bad |= (block_max(m_raw, sb) >= INF16 ? 1u : 0u) << sb;
       tiny_rows = group_and_u32<TPR>(tiny_rows);      // rows tiny in every lane of their group
       need_norms = __any(tiny_rows != 0);             // rare
     }
@@ -1145,6 +1173,14 @@ hipError_t launch_km_mean_static(const void *k, Strides ks, void *km, int B, int
   hipError_t e = hipGetDevice(&dev);
   if (e != hipSuccess) return e;
   if (dev < 0 || dev >= MAX_DEV) return hipErrorInvalidDevice;
+  // The array's address is looked up for, and only valid on, the CURRENT device: a stream that belongs to another GPU
+  // would run the kernels there with this GPU's address.  (The null stream always belongs to the current device.)
+  if (st != nullptr) {
+    hipDevice_t sdev = -1;
+    e = hipStreamGetDevice(st, &sdev);
+    if (e != hipSuccess) return e;
+    if ((int)sdev != dev) return hipErrorInvalidDevice;
+  }
   void *ptr = scratch_of_device[dev].load(std::memory_order_acquire);
   if (ptr == nullptr) {
     // first call on this device (the device is current): resolve this GPU's copy of the array

@@ -37,6 +37,7 @@ __global__ __launch_bounds__(256) void v_absmax_kernel(const uint16_t *__restric
   // is taken on the 16-bit magnitude patterns (which order like the magnitudes), two per instruction, and only the
   // result is converted.
   typedef unsigned short u16x2_t __attribute__((ext_vector_type(2)));
+  constexpr uint32_t INF16 = DT == 1 ? 0x7f80u : 0x7c00u;
   uint32_t mp[4] = {0, 0, 0, 0};
 #pragma unroll 4
   for (int row = row0 + r; row < row1; row += RPP) {
@@ -46,6 +47,24 @@ __global__ __launch_bounds__(256) void v_absmax_kernel(const uint16_t *__restric
     for (int j = 0; j < 4; j++)
       mp[j] = __builtin_bit_cast(uint32_t, __builtin_elementwise_max(__builtin_bit_cast(u16x2_t, mp[j]),
                                                                       __builtin_bit_cast(u16x2_t, w[j] & 0x7fff7fffu)));
+  }
+  // A NaN pattern lies above the infinity pattern and would win the maximum, whereas the reference's fmaxf / fminf
+  // (fused.cu:120-123) ignore NaN: only the NaN elements themselves are poisoned, not their channel's scale.  The
+  // common case pays one test; a thread that met a NaN goes over its rows again with the NaN patterns taken as zero.
+  if (max(max(mp[0] & 0xffffu, mp[0] >> 16), max(mp[1] & 0xffffu, mp[1] >> 16)) > INF16 ||
+      max(max(mp[2] & 0xffffu, mp[2] >> 16), max(mp[3] & 0xffffu, mp[3] >> 16)) > INF16) {
+    mp[0] = mp[1] = mp[2] = mp[3] = 0;
+    for (int row = row0 + r; row < row1; row += RPP) {
+      const uint4 q = *(const uint4 *)(base + (size_t)row * vs.sn);
+      const uint32_t w[4] = {q.x, q.y, q.z, q.w};
+#pragma unroll
+      for (int j = 0; j < 4; j++) {
+        uint32_t lo = w[j] & 0x7fffu, hi = (w[j] >> 16) & 0x7fffu;
+        lo = lo > INF16 ? 0u : lo;
+        hi = hi > INF16 ? 0u : hi;
+        mp[j] = max(mp[j] & 0xffffu, lo) | (max(mp[j] >> 16, hi) << 16);
+      }
+    }
   }
   float m[8];
 #pragma unroll

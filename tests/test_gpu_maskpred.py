@@ -246,3 +246,49 @@ def test_helper_wrappers_of_the_reference_utils():
     assert torch.equal(p2, want[0]) and torch.equal(s2, want[1])
     with pytest.raises(ValueError):
         utils.get_quant(x, None, 32)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("D", [64, 128])
+def test_a_nan_poisons_its_own_element_not_the_scale(dtype, D):
+    """The reference's maxima ignore NaN (fmaxf / fminf in csrc/fused/fused.cu:120-123, tl.max = maxnum in
+    spas_sage_attn/utils.py:140, 206): one NaN in V or Q leaves the channel / block scale that of the other elements and
+    only its own code is affected (FP8 NaN, INT8 0); the block that holds it is never "similar"."""
+    tag = tag_of(dtype)
+    B, H, N = 1, 2, 700
+    v = rand_T((B, H, N, D), dtype, 11)
+    q = rand_T((B, H, N, D), dtype, 12)
+    v[0, 1, 333, 5] = float("nan")
+    q[0, 0, 200, 7] = float("nan")                      # block 1 of head 0 (rows 128..255), 32-row group 6
+    v8, vs = _lib.v_quant_fp8(v)
+    ref8, refs = vq.v_quant_fp8(vq.to_fp16(to_np(v)))
+    assert np.array_equal(vs.cpu().numpy().view(np.uint32), refs.view(np.uint32)) and np.isfinite(refs).all()
+    got8 = v8_natural(v8, N)
+    nan_at = np.zeros(got8.shape, dtype=bool)
+    nan_at[0, 1, 333, 5] = True
+    assert np.array_equal(got8[~nan_at], ref8[:, :, :N][~nan_at])
+    # the NaN element itself: an e4m3 NaN code (sign bit free: 0x7f or 0xff) on both sides, and nowhere else
+    assert (got8[nan_at] & 0x7F) == 0x7F and (ref8[:, :, :N][nan_at] & 0x7F) == 0x7F, (got8[nan_at], ref8[:, :, :N][nan_at])
+    assert ((got8[0, 1, :, 5] & 0x7F) == 0x7F).sum() == 1
+    thr = torch.full((H,), 0.2, dtype=torch.float32, device="cuda")
+    for quant_rows, with_pool in ((128, True), (32, True), (128, False)):
+        pool, sim, xq, scale = _lib.pool_sim_quant(q, None, 128, thr, with_pool=with_pool, quant_rows=quant_rows)
+        ref = mp.pool_sim_quant(to_np(q), None, 128, thr.cpu().numpy(), tag, with_pool=with_pool, quant_rows=quant_rows)
+        assert np.array_equal(xq.cpu().numpy(), ref["q"]) and xq[0, 0, 200, 7] == 0
+        assert np.array_equal(scale.cpu().numpy().view(np.uint32), ref["scale"].view(np.uint32))
+        assert np.isfinite(ref["scale"]).all()
+        if with_pool:
+            assert np.array_equal(sim.cpu().numpy(), ref["sim"]) and not ref["sim"][0, 0, 1]
+            gp = to_np(pool)
+            assert np.array_equal(np.isnan(gp), np.isnan(ref["pool"])) and np.isnan(gp[0, 0, 1, 7])
+            ok = ~np.isnan(gp)
+            assert np.array_equal(gp[ok], ref["pool"][ok])
+    # a negative similarity threshold decides the flag without the normalised rows: the NaN still clears it
+    _, sim, _, _ = _lib.pool_sim_quant(q, None, 128, torch.full((H,), -0.1, dtype=torch.float32, device="cuda"))
+    assert not bool(sim[0, 0, 1]) and bool(sim[0, 0, 0])
+    # K path (mean subtracted): the NaN reaches the column mean of its channel, as in the reference
+    km = _lib.km_mean(q)
+    _, _, kq, ks = _lib.pool_sim_quant(q, km, 64, thr)
+    refk = mp.pool_sim_quant(to_np(q), mp.km_mean(to_np(q), tag), 64, thr.cpu().numpy(), tag)
+    assert np.array_equal(kq.cpu().numpy(), refk["q"])
+    assert np.array_equal(ks.cpu().numpy().view(np.uint32), refk["scale"].view(np.uint32))

@@ -107,3 +107,16 @@ attn.hip:2:1: remark:     VGPRs Spill: 6 [-Rpass-analysis=kernel-resource-usage]
 """
     bad = build._spill_report(log)
     assert len(bad) == 2 and all(b.startswith("kern_b") for b in bad)
+
+
+def test_build_names_the_compiler_it_was_validated_with(monkeypatch):
+    """attn.hip / dense.hip wait for some inline-asm LDS reads in a later statement; the build refuses (or, with the
+    override, warns about) a compiler whose generated code has not been inspected for those windows."""
+    from spargeattn_amd import build as b
+    ok, version = b.check_compiler()
+    assert ok and "roc-7.2.0" in version                      # the toolchain of this image
+    monkeypatch.setattr(b, "_compiler_version", lambda: "AMD clang version 99.0.0 (roc-99.0.0)")
+    assert b.check_compiler() == (False, "AMD clang version 99.0.0 (roc-99.0.0)")
+    monkeypatch.delenv("SPARGEATTN_AMD_ALLOW_UNVALIDATED_COMPILER", raising=False)
+    with pytest.raises(RuntimeError, match="not a validated version"):
+        b.build(verbose=False)
