@@ -1,9 +1,17 @@
-"""ctypes binding of libspargeattn_amd.so (the C ABI in include/spargeattn_amd.h).
+"""Bindings of libspargeattn_amd.so (the C ABI in include/spargeattn_amd.h).
 
-PyTorch is used for device memory and streams only: every wrapper below hands raw
-``data_ptr()`` addresses and the current HIP stream to the library.  There is no CPU or
-eager fallback: if the library is missing, or no GPU tensor is given, the call raises.
+Two interchangeable bindings sit under the stage wrappers of this module:
+
+* ``"ctypes"`` (default, nothing to compile beyond the library): PyTorch supplies device memory and the current
+  stream, the wrappers hand raw ``data_ptr()`` addresses to the C functions;
+* ``"torch"``: the PyTorch extension ``libspargeattn_amd_torch.so`` (csrc/torch_ext.cpp), whose operators are
+  registered as ``torch.ops.spargeattn_amd.*`` with meta kernels and do their own TORCH_CHECKs, allocation and stream
+  lookup in C++ - the form the reference's pybind modules have (csrc/qattn/pybind.cpp:20-36).
+
+Select with ``set_binding("torch")`` or the environment variable ``SPARGEATTN_AMD_BINDING``.  There is no CPU or eager
+fallback in either: if the library is missing, or no GPU tensor is given, the call raises.
 """
+import contextlib
 import ctypes
 import os
 
@@ -11,6 +19,7 @@ import torch
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libspargeattn_amd.so")
+TORCH_EXT_PATH = os.path.join(_HERE, "libspargeattn_amd_torch.so")
 
 SPG_OK, SPG_ERR_INVALID, SPG_ERR_UNSUPPORTED, SPG_ERR_HIP = 0, 1, 2, 3
 SPG_F16, SPG_BF16 = 0, 1
@@ -38,10 +47,46 @@ SIGNATURES = {
 }
 
 _lib = None
+_ops = None          # torch.ops.spargeattn_amd once the extension is loaded
+_binding = None      # "ctypes" or "torch"; resolved on first use from SPARGEATTN_AMD_BINDING
 
 
 class SpargeError(RuntimeError):
     pass
+
+
+def set_binding(name):
+    """Route the stage wrappers through the ctypes binding ("ctypes") or the PyTorch extension ("torch")."""
+    global _binding
+    if name not in ("ctypes", "torch"):
+        raise ValueError(f"unknown binding {name!r}: expected 'ctypes' or 'torch'")
+    if name == "torch":
+        load_torch_ext()
+    _binding = name
+
+
+def get_binding():
+    global _binding
+    if _binding is None:
+        set_binding(os.environ.get("SPARGEATTN_AMD_BINDING", "ctypes"))
+    return _binding
+
+
+def _torch():
+    """torch.ops.spargeattn_amd when the torch binding is selected, else None."""
+    return _ops if get_binding() == "torch" else None
+
+
+def load_torch_ext():
+    """Load the PyTorch extension (once) and return torch.ops.spargeattn_amd.  Raises if it has not been built."""
+    global _ops
+    if _ops is None:
+        load()                                   # the extension links against the C-ABI library beside it
+        if not os.path.exists(TORCH_EXT_PATH):
+            raise SpargeError(f"{TORCH_EXT_PATH} not found: build it with `python -m spargeattn_amd.build`.")
+        torch.ops.load_library(TORCH_EXT_PATH)
+        _ops = torch.ops.spargeattn_amd
+    return _ops
 
 
 def load():
@@ -129,6 +174,8 @@ _MASK_KIND = {
 def km_mean(k):
     """k (B,H,N,D) -> km (B,H,1,D), same dtype."""
     _dev_strided(k)
+    if _torch() is not None:
+        return _ops.km_mean(k)
     B, H, N, D = k.shape
     lib = load()
     km = torch.empty((B, H, 1, D), dtype=k.dtype, device=k.device)
@@ -148,6 +195,10 @@ def pool_sim_quant(x, km, block, simthreshd1=None, with_pool=True, stream=None, 
     quant_rows = block if quant_rows is None else int(quant_rows)
     if quant_rows <= 0 or block % quant_rows:
         raise ValueError(f"quant_rows ({quant_rows}) must divide the block size ({block})")
+    if _torch() is not None:
+        with torch.cuda.stream(stream) if stream is not None else contextlib.nullcontext():
+            pool, sim, xq, scale = _ops.pool_sim_quant(x, km, block, simthreshd1 if with_pool else None, with_pool, quant_rows)
+        return (pool, sim, xq, scale) if with_pool else (None, None, xq, scale)
     xq = torch.empty((B, H, N, D), dtype=torch.int8, device=x.device)
     scale = torch.empty((B, H, nb * (block // quant_rows)), dtype=torch.float32, device=x.device)
     pool = sim = None
@@ -170,6 +221,10 @@ def block_select(pool_q, sim_q, pool_k, sim_k, topk=None, cdfthreshd=None, is_ca
     for t in (topk, cdfthreshd):
         if t is not None and t.numel() != H:
             raise RuntimeError(f"per-head hyper-parameter has {t.numel()} entries, expected {H}")
+    if _torch() is not None:
+        lut, valid, bmap = _ops.block_select(pool_q, sim_q, pool_k, sim_k, topk, cdfthreshd, bool(is_causal),
+                                             bool(attention_sink), bool(return_map))
+        return lut, valid, (bmap if return_map else None)
     lut = torch.empty((B, H, nq, nk), dtype=torch.int32, device=pool_q.device)
     valid = torch.empty((B, H, nq), dtype=torch.int32, device=pool_q.device)
     bmap = torch.empty((B, H, nq, nk), dtype=torch.bool, device=pool_q.device) if return_map else None
@@ -183,6 +238,8 @@ def map_to_lut(block_map):
     _dev(block_map)
     if block_map.dtype not in _MASK_KIND:
         raise RuntimeError(f"unsupported mask dtype {block_map.dtype}")
+    if _torch() is not None:
+        return tuple(_ops.map_to_lut(block_map))
     B, H, nq, nk = block_map.shape
     lut = torch.empty((B, H, nq, nk), dtype=torch.int32, device=block_map.device)
     valid = torch.empty((B, H, nq), dtype=torch.int32, device=block_map.device)
@@ -193,6 +250,9 @@ def map_to_lut(block_map):
 def v_quant_fp8(v, stream=None):
     """v (B,H,N,D) fp16/bf16 -> (v8 uint8 codes in tile layout (B,H,nk,D,64), v_scale (B,H,D) float32)."""
     _dev_strided(v)
+    if _torch() is not None:
+        with torch.cuda.stream(stream) if stream is not None else contextlib.nullcontext():
+            return tuple(_ops.v_quant_fp8(v))
     B, H, N, D = v.shape
     nk = (N + 63) // 64
     v8 = torch.empty((B, H, nk, D, 64), dtype=torch.uint8, device=v.device)
@@ -273,6 +333,10 @@ def block_sparse_attn(q8, k8, v8, out, lut, valid, pvthreshd, q_scale, k_scale, 
     B, H, Hkv, N, Nk, D = _check_attn_shapes(q8, k8, v8, lut, valid, q_scale, k_scale, v_scale, qk_quant_gran)
     if tuple(out.shape) != (B, H, N, D) or pvthreshd.numel() != H:
         raise RuntimeError("out must have q's shape and pvthreshd one entry per query head")
+    if _torch() is not None:
+        pvc = _ops.block_sparse_attn(q8, k8, v8, out, lut, valid, pvthreshd, q_scale, k_scale, v_scale, float(sm_scale),
+                                     bool(is_causal), qk_quant_gran, int(pv_mode), bool(return_pv_count))
+        return pvc if return_pv_count else None
     pvc = torch.zeros((B, H, 4 * ((N + 127) // 128)), dtype=torch.int32, device=q8.device) if return_pv_count else None
     _check(load().spg_block_sparse_attn(_p(q8), _p(k8), _p(v8), _p(out), _st(out), _dt(out), _p(lut), _p(valid), _p(pvthreshd),
                                         _p(q_scale), _p(k_scale), _p(v_scale), B, H, Hkv, N, Nk, D, float(sm_scale),
@@ -283,6 +347,9 @@ def block_sparse_attn(q8, k8, v8, out, lut, valid, pvthreshd, q_scale, k_scale, 
 def v_tiles_f16_swizzled(v, stream=None):
     """v (B,H,N,D) fp16/bf16 -> (B,H,nk,D,64) fp16 V^T tiles, chunk-swizzled, the operand of block_sparse_attn_f16v."""
     _dev_strided(v)
+    if _torch() is not None:
+        with torch.cuda.stream(stream) if stream is not None else contextlib.nullcontext():
+            return _ops.v_tiles_f16(v)
     B, H, N, D = v.shape
     nk = (N + 63) // 64
     vt = torch.empty((B, H, nk, D, 64), dtype=torch.float16, device=v.device)
@@ -308,6 +375,10 @@ def block_sparse_attn_f16v(q8, k8, vt, out, lut, valid, pvthreshd, q_scale, k_sc
     B, H, Hkv, N, Nk, D = _check_attn_shapes(q8, k8, vt, lut, valid, q_scale, k_scale, None, qk_quant_gran)
     if tuple(out.shape) != (B, H, N, D) or pvthreshd.numel() != H:
         raise RuntimeError("out must have q's shape and pvthreshd one entry per query head")
+    if _torch() is not None:
+        pvc = _ops.block_sparse_attn_f16v(q8, k8, vt, out, lut, valid, pvthreshd, q_scale, k_scale, float(sm_scale),
+                                          bool(is_causal), qk_quant_gran, int(pv_mode), bool(return_pv_count))
+        return pvc if return_pv_count else None
     pvc = torch.zeros((B, H, 4 * ((N + 127) // 128)), dtype=torch.int32, device=q8.device) if return_pv_count else None
     _check(load().spg_block_sparse_attn_f16v(_p(q8), _p(k8), _p(vt), _p(out), _st(out), _dt(out), _p(lut), _p(valid),
                                              _p(pvthreshd), _p(q_scale), _p(k_scale), B, H, Hkv, N, Nk, D, float(sm_scale),
@@ -322,6 +393,8 @@ def dense_attn_f16(q, k, vt, sm_scale, is_causal=False, out=None):
     B, H, N, D = q.shape
     if out is None:
         out = torch.empty_like(q)
+    if _torch() is not None:
+        return _ops.dense_attn_f16(q, k, vt, out, float(sm_scale), bool(is_causal))
     _check(load().spg_dense_attn_f16(_p(q), _p(k), _p(vt), _p(out), B, H, N, D, float(sm_scale),
                                      int(bool(is_causal)), _stream()))
     return out
@@ -331,6 +404,8 @@ def selftest_fp8_pack(x, saturate=True):
     """float32 GPU tensor (size a multiple of 4) -> uint8 e4m3 codes from the attention kernel's pack."""
     _dev(x)
     assert x.dtype == torch.float32 and x.numel() % 4 == 0
+    if _torch() is not None:
+        return _ops.selftest_fp8_pack(x, bool(saturate))
     codes = torch.empty(x.numel(), dtype=torch.uint8, device=x.device)
     _check(load().spg_selftest_fp8_pack(_p(x), _p(codes), x.numel(), int(bool(saturate)), _stream()))
     return codes.view(x.shape)
@@ -339,5 +414,7 @@ def selftest_fp8_pack(x, saturate=True):
 def selftest_division(n_divisors, seed=1):
     """Returns (comparisons, mismatches) of the shared-reciprocal division against the hardware's IEEE division."""
     counts = torch.zeros(2, dtype=torch.int64, device="cuda")
+    if _torch() is not None:
+        return tuple(int(c) for c in _ops.selftest_division(counts, int(n_divisors), int(seed)).cpu())
     _check(load().spg_selftest_division(_p(counts), int(n_divisors), int(seed), _stream()))
     return tuple(int(c) for c in counts.cpu())

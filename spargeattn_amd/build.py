@@ -107,5 +107,32 @@ def build(verbose=True):
     return LIB
 
 
+TORCH_EXT_LIB = os.path.join(HERE, "libspargeattn_amd_torch.so")
+
+
+def build_torch_ext(verbose=True):
+    """csrc/torch_ext.cpp -> libspargeattn_amd_torch.so: the torch.ops.spargeattn_amd.* registrations over the C ABI.
+    Host code only (no kernel lives in the shim); links against libspargeattn_amd.so beside it and against torch."""
+    import torch
+    from torch.utils import cpp_extension as ce
+    tlib = os.path.join(os.path.dirname(torch.__file__), "lib")
+    obj = os.path.join(CSRC, "torch_ext.o")
+    cmd = [HIPCC, "-x", "c++", "-O2", "-fPIC", "-std=c++17", "-fvisibility=hidden", "-Wno-unused-command-line-argument",
+           "-D__HIP_PLATFORM_AMD__=1", "-DUSE_ROCM=1",
+           f"-D_GLIBCXX_USE_CXX11_ABI={int(torch._C._GLIBCXX_USE_CXX11_ABI)}",
+           *[f"-I{p}" for p in ce.include_paths()], "-I/opt/rocm/include",
+           "-c", os.path.join(CSRC, "torch_ext.cpp"), "-o", obj]
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    if r.returncode != 0:
+        raise RuntimeError(f"torch extension failed to compile:\n{' '.join(cmd)}\n{r.stderr[-6000:]}")
+    cmd = [HIPCC, "-shared", "-fPIC", "-o", TORCH_EXT_LIB, obj, f"-L{HERE}", "-lspargeattn_amd", "-Wl,-rpath,$ORIGIN",
+           f"-L{tlib}", "-lc10", "-lc10_hip", "-ltorch_cpu", "-ltorch_hip", "-ltorch"]
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    if r.returncode != 0:
+        raise RuntimeError(f"torch extension failed to link:\n{r.stderr[-6000:]}")
+    return TORCH_EXT_LIB
+
+
 if __name__ == "__main__":
     print(build())
+    print(build_torch_ext())
