@@ -32,6 +32,11 @@ SOURCES = {
 # when any kernel of these files uses scratch memory or spills a vector register.  (Scalar registers parked in the
 # lanes of a vector register - "SGPRs Spill" - never touch memory or the registers those reads write, and are allowed.)
 NO_SPILL = {"attn.hip", "dense.hip"}
+# Kernels of those files that issue EVERY inline-asm LDS read together with its wait (no window in which a register is
+# in flight) may use scratch: the FP16-PV attention variants (template argument PV16 = true, "Lb1" in the mangled
+# name), whose masked tail loop parks a few registers there.
+SPILL_EXEMPT = ("block_sparse_attn_kernelILi128ELi0ELb1", "block_sparse_attn_kernelILi128ELi1ELb1",
+                "block_sparse_attn_kernelILi64ELi0ELb1", "block_sparse_attn_kernelILi64ELi1ELb1")
 RESOURCE_REMARKS = "-Rpass-analysis=kernel-resource-usage"
 # The same kernels issue some LDS reads through inline asm and wait for them in a LATER asm statement (the reads run
 # under matrix instructions).  In between, the compiler believes the destination registers are already written; the
@@ -61,7 +66,7 @@ def _spill_report(stderr):
         for key in ("ScratchSize [bytes/lane]:", "VGPRs Spill:"):
             if key in line:
                 value = line.split(key)[1].split("[")[0].strip()
-                if value != "0":
+                if value != "0" and not any(tag in (name or "") for tag in SPILL_EXEMPT):
                     bad.append(f"{name}: {key} {value}")
     return bad
 

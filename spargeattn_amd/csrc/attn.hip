@@ -125,12 +125,12 @@ __device__ __forceinline__ int v_swz(int row) { return (row >> 2) & 3; }
 // PV16 = false: V^T tiles are e4m3 (64 bytes per channel row), P is packed to e4m3 with the +8.807 exponent offset and
 //               the denominator sums the un-rounded P (the SageAttention2 kernel, sm89.cuh).
 // PV16 = true:  V^T tiles are fp16 (128 bytes per channel row, 16-byte chunks swizzled by slot = chunk ^ ((d >> 1) & 7)), P is
-//               rounded to fp16 and the denominator sums the ROUNDED P (the SageAttention1 kernel with the row sum on
-//               the matrix unit, qk_int_sv_f16_cuda_sm80.cuh:339-368, attn_utils.cuh:599-626).  The PV product is
+//               rounded to fp16 and the denominator sums the ROUNDED P in binary32 (what the SageAttention1 kernel's row
+//               sum on the tensor cores computes, qk_int_sv_f16_cuda_sm80.cuh:339-368, attn_utils.cuh:599-626).  The PV product is
 //               accumulated in fp32; the reference accumulates each 64-key block in fp16 before adding it to its fp32
 //               accumulator (attn_utils.cuh:683-751), a rounding this kernel does not reproduce.
 template <int D, int ODT, bool PV16>
-__global__ __launch_bounds__(256, PV16 ? 2 : 3) void block_sparse_attn_kernel(const AttnParams p) {
+__global__ __launch_bounds__(256, 3) void block_sparse_attn_kernel(const AttnParams p) {
   constexpr int KS = D / 32;        // k-steps of the int8 MFMA
   constexpr int NDT = D / 32;       // 32-channel output tiles
   constexpr int TILE = 64 * D;      // bytes of one K tile
@@ -138,8 +138,11 @@ __global__ __launch_bounds__(256, PV16 ? 2 : 3) void block_sparse_attn_kernel(co
   constexpr int CPR = D / 16;       // 16-byte chunks per K row
   constexpr int WL = D / 64;        // global_load_lds instructions per wave per K tile (TILE / 1024 / 4)
   constexpr int WLV = VTILE / 4096; // ... per V^T tile
-  constexpr int NBUF = 3;
-  // LDS: K ring [NBUF][TILE] | V^T ring [NBUF][TILE] | votes
+  // Tile rings.  FP8 PV: three slots each, the tiles of block it+2 are requested while block it is computed.
+  // FP16 PV (tiles twice as large): two slots each, so that three workgroups still share a CU (48 KiB): the K tile of
+  // block it+2 goes to the slot block it's K tile just left, the V^T tile of block it+1 to the slot of block it-1.
+  constexpr int NBUF = PV16 ? 2 : 3;
+  // LDS: K ring [NBUF][TILE] | V^T ring [NBUF][VTILE] | votes
   __shared__ __align__(1024) unsigned char smem[NBUF * (TILE + VTILE)];
   // PV-skip vote of the per-block mode: a wavefront that votes "skip" stamps the iteration number into its slot; a slot
   // that does not hold the current iteration number means "compute".  Only "skip" votes are written (they are rare at the
@@ -214,25 +217,15 @@ __global__ __launch_bounds__(256, PV16 ? 2 : 3) void block_sparse_attn_kernel(co
   const int last_partial_blk = (Nk % 64) ? p.nk - 1 : -1;   // the only block with rows beyond Nk
   typedef __attribute__((address_space(3))) void *lds_ptr_t;
   typedef const __attribute__((address_space(1))) void *glb_ptr_t;
-#define SPG_LOAD_TILES(BLK, BUFOFF)                                                                           \
+#define SPG_LOAD_K_(BLK, KOFF)   /* inside a scope that holds SPG_LANE_OFFSETS() */                            \
   {                                                                                                           \
-    SPG_LANE_OFFSETS()                                                                                        \
     const int8_t *kb_ = kbase + (size_t)(BLK) * TILE;                                                         \
-    const uint8_t *vb_ = vbase + (size_t)(BLK) * VTILE;                                                       \
-    unsigned char *lk_ = sKr + (BUFOFF) + WL * wave * 1024;                                                   \
-    unsigned char *lv_ = sVr + (PV16 ? 2 * (BUFOFF) : (BUFOFF)) + WLV * wave * 1024;                          \
+    unsigned char *lk_ = sKr + (KOFF) + WL * wave * 1024;                                                     \
     if ((BLK) != last_partial_blk) {                                                                          \
       /* the loads of one tile back to back: they share the LDS base register (M0) */                          \
       __builtin_amdgcn_global_load_lds((glb_ptr_t)(kb_ + k_lane), (lds_ptr_t)lk_, 16, 0, 0);                  \
       if constexpr (WL == 2)                                                                                  \
         __builtin_amdgcn_global_load_lds((glb_ptr_t)(kb_ + k_lane), (lds_ptr_t)lk_, 16, 1024, 0);             \
-      __builtin_amdgcn_global_load_lds((glb_ptr_t)(vb_ + v_lane), (lds_ptr_t)lv_, 16, 0, 0);                  \
-      if constexpr (WLV >= 2)                                                                                 \
-        __builtin_amdgcn_global_load_lds((glb_ptr_t)(vb_ + v_lane), (lds_ptr_t)lv_, 16, 1024, 0);             \
-      if constexpr (WLV == 4) {                                                                               \
-        __builtin_amdgcn_global_load_lds((glb_ptr_t)(vb_ + v_lane), (lds_ptr_t)lv_, 16, 2048, 0);             \
-        __builtin_amdgcn_global_load_lds((glb_ptr_t)(vb_ + v_lane), (lds_ptr_t)lv_, 16, 3072, 0);             \
-      }                                                                                                       \
     } else {                                                                                                  \
       /* rows beyond Nk are clamped to row Nk-1: their scores are masked, their V rows are zero */              \
       const int rows_ok_ = Nk - (BLK) * 64;                                                                    \
@@ -242,10 +235,24 @@ __global__ __launch_bounds__(256, PV16 ? 2 : 3) void block_sparse_attn_kernel(co
         const uint32_t ko_ = row_ * D + (((pos % CPR) ^ k_swz<D>(pos / CPR)) * 16u);                          \
         __builtin_amdgcn_global_load_lds((glb_ptr_t)(kb_ + ko_), (lds_ptr_t)(lk_ + u * 1024), 16, 0, 0);      \
       }                                                                                                       \
-      _Pragma("unroll") for (int u = 0; u < WLV; u++)                                                         \
-        __builtin_amdgcn_global_load_lds((glb_ptr_t)(vb_ + v_lane + u * 1024), (lds_ptr_t)(lv_ + u * 1024), 16, 0, 0); \
     }                                                                                                         \
   }
+#define SPG_LOAD_V_(BLK, VOFF)                                                                                \
+  {                                                                                                           \
+    const uint8_t *vb_ = vbase + (size_t)(BLK) * VTILE;                                                       \
+    unsigned char *lv_ = sVr + (VOFF) + WLV * wave * 1024;                                                    \
+    __builtin_amdgcn_global_load_lds((glb_ptr_t)(vb_ + v_lane), (lds_ptr_t)lv_, 16, 0, 0);                    \
+    if constexpr (WLV >= 2)                                                                                   \
+      __builtin_amdgcn_global_load_lds((glb_ptr_t)(vb_ + v_lane), (lds_ptr_t)lv_, 16, 1024, 0);               \
+    if constexpr (WLV == 4) {                                                                                 \
+      __builtin_amdgcn_global_load_lds((glb_ptr_t)(vb_ + v_lane), (lds_ptr_t)lv_, 16, 2048, 0);               \
+      __builtin_amdgcn_global_load_lds((glb_ptr_t)(vb_ + v_lane), (lds_ptr_t)lv_, 16, 3072, 0);               \
+    }                                                                                                         \
+  }
+#define SPG_LOAD_K(BLK, KOFF) { SPG_LANE_OFFSETS() (void)v_lane; SPG_LOAD_K_(BLK, KOFF) }
+#define SPG_LOAD_V(BLK, VOFF) { SPG_LANE_OFFSETS() (void)k_lane; (void)pos0; SPG_LOAD_V_(BLK, VOFF) }
+// FP8 PV: both tiles of one block into ring slot offset BUFOFF (in K-tile units)
+#define SPG_LOAD_TILES(BLK, BUFOFF) { SPG_LANE_OFFSETS() SPG_LOAD_K_(BLK, BUFOFF) SPG_LOAD_V_(BLK, BUFOFF) }
 
   // MFMA row i of key tile kt carries key 32*((i>>2)&1) + 16*kt + 4*(i>>3) + (i&3); rows krow0 and krow0+16 have
   // the same swizzle, so tile 1's operand sits 16 rows (16*D bytes) after tile 0's.
@@ -262,9 +269,8 @@ __global__ __launch_bounds__(256, PV16 ? 2 : 3) void block_sparse_attn_kernel(co
   const uint32_t v_rd16 = (uint32_t)(r * 128 + (((4 * hh) ^ ((r >> 1) & 7)) * 16));
 
   float m = SPG_NEG_BIG;
-  // d = 1.0 initially (sm89.cuh:172).  FP8 path: each half-lane sums its own 32 keys, so only one of the two starts at 1;
-  // FP16 path: both half-lanes hold the full row sum.
-  float dsum = (PV16 || hh == 0) ? 1.0f : 0.0f;
+  // d = 1.0 initially (sm89.cuh:172).  Each half-lane sums its own 32 keys, so only one of the two starts at 1.
+  float dsum = hh == 0 ? 1.0f : 0.0f;
   v16f O[NDT];
 #pragma unroll
   for (int dt = 0; dt < NDT; dt++)
@@ -279,8 +285,14 @@ __global__ __launch_bounds__(256, PV16 ? 2 : 3) void block_sparse_attn_kernel(co
   int blk2 = blk1 + (nv > 2 ? lutc[2] : 0);
   int d3 = nv > 3 ? lutc[3] : 0;
   float ksc = kscale[blk], ksc1 = kscale[blk1];
-  SPG_LOAD_TILES(blk, 0);
-  if (nv > 1) SPG_LOAD_TILES(blk1, TILE);
+  if constexpr (PV16) {
+    SPG_LOAD_K(blk, 0);
+    SPG_LOAD_V(blk, 0);
+    if (nv > 1) SPG_LOAD_K(blk1, TILE);           // the V^T tile of block 1 follows behind the first barrier
+  } else {
+    SPG_LOAD_TILES(blk, 0);
+    if (nv > 1) SPG_LOAD_TILES(blk1, TILE);
+  }
   uint32_t bufoff = 0;                     // LDS ring offset of block it
 
   // The INT8 accumulators do not start at zero but at the bit pattern 0x3E22F983 - the float 1/(2 pi), which the
@@ -329,8 +341,12 @@ __global__ __launch_bounds__(256, PV16 ? 2 : 3) void block_sparse_attn_kernel(co
         if constexpr (HK == 2) lds_read_4x128_wait<SO, SO + 16 * D>(a0[0], a1[0], a0[1], a1[1], kaddr_c[0] + bo, kaddr_c[1] + bo);
         else lds_read_2x128_wait<SO, SO + 16 * D>(a0[0], a1[0], kaddr_c[0] + bo, kaddr_c[0] + bo);
       }
+      // second group: in flight under the first group's products (FP8 PV); the FP16-PV variant reads it afterwards, into
+      // the first group's registers, which is what lets it keep three wavefronts per SIMD
+      if constexpr (!PV16) {
 #pragma unroll
-      for (int ks = HK; ks < KS; ks++) read_k(ks);
+        for (int ks = HK; ks < KS; ks++) read_k(ks);
+      }
       // the first product of each chain, with the inline constant as its C operand (the compiler would otherwise keep
       // the constant in sixteen registers); the products that follow accumulate onto these and are ordinary builtins,
       // which the other chain's product always separates from their predecessor
@@ -342,11 +358,21 @@ __global__ __launch_bounds__(256, PV16 ? 2 : 3) void block_sparse_attn_kernel(co
         S0 = __builtin_amdgcn_mfma_i32_32x32x32_i8(a0[ks], qreg[ks], S0, 0, 0, 0);
         S1 = __builtin_amdgcn_mfma_i32_32x32x32_i8(a1[ks], qreg[ks], S1, 0, 0, 0);
       }
-      if constexpr (HK == 2) lds_wait4(a0[2], a1[2], a0[3], a1[3]); else lds_wait2(a0[1], a1[1]);
+      if constexpr (PV16) {
+        if constexpr (HK == 2) lds_read_4x128_wait<0, 16 * D>(a0[0], a1[0], a0[1], a1[1], kaddr_c[2] + bufoff, kaddr_c[3] + bufoff);
+        else lds_read_2x128_wait<0, 16 * D>(a0[0], a1[0], kaddr_c[1] + bufoff, kaddr_c[1] + bufoff);
 #pragma unroll
-      for (int ks = HK; ks < KS; ks++) {
-        S0 = __builtin_amdgcn_mfma_i32_32x32x32_i8(a0[ks], qreg[ks], S0, 0, 0, 0);
-        S1 = __builtin_amdgcn_mfma_i32_32x32x32_i8(a1[ks], qreg[ks], S1, 0, 0, 0);
+        for (int ks = HK; ks < KS; ks++) {
+          S0 = __builtin_amdgcn_mfma_i32_32x32x32_i8(a0[ks - HK], qreg[ks], S0, 0, 0, 0);
+          S1 = __builtin_amdgcn_mfma_i32_32x32x32_i8(a1[ks - HK], qreg[ks], S1, 0, 0, 0);
+        }
+      } else {
+        if constexpr (HK == 2) lds_wait4(a0[2], a1[2], a0[3], a1[3]); else lds_wait2(a0[1], a1[1]);
+#pragma unroll
+        for (int ks = HK; ks < KS; ks++) {
+          S0 = __builtin_amdgcn_mfma_i32_32x32x32_i8(a0[ks], qreg[ks], S0, 0, 0, 0);
+          S1 = __builtin_amdgcn_mfma_i32_32x32x32_i8(a1[ks], qreg[ks], S1, 0, 0, 0);
+        }
       }
     }
 
@@ -426,7 +452,14 @@ __global__ __launch_bounds__(256, PV16 ? 2 : 3) void block_sparse_attn_kernel(co
         compute = !(sSkipAt[it & 1][0] == it && sSkipAt[it & 1][1] == it && sSkipAt[it & 1][2] == it &&
                     sSkipAt[it & 1][3] == it);
     }
-    if (!TAIL || it + 2 < nv) {
+    if constexpr (PV16) {
+      // two-slot rings: every wavefront is past its reads of K slot it % 2 (this block's scores) and of V^T slot
+      // (it + 1) % 2 (the previous block's P.V product)
+      SPG_LANE_OFFSETS()
+      (void)pos0;
+      if (!TAIL || it + 2 < nv) SPG_LOAD_K_(blk2, bufoff);
+      if (!TAIL || it + 1 < nv) SPG_LOAD_V_(blk1, 2 * (bufoff ^ (uint32_t)TILE));
+    } else if (!TAIL || it + 2 < nv) {
       if constexpr (CS) {
         SPG_LOAD_TILES(blk2, ((SLOT + 2) % 3) * TILE);
       } else {
@@ -501,40 +534,38 @@ __global__ __launch_bounds__(256, PV16 ? 2 : 3) void block_sparse_attn_kernel(co
             pb16[s4][j + 1] = ph[1];
           }
         {
-          // row sums of the ROUNDED P on the matrix unit, as the reference does (rowsum_f16f16f32, attn_utils.cuh:614):
-          // ones (32 x 16) . P^T gives, in every row, the sum over the 16 keys of the step for each query column
-          const h8 ones = {(_Float16)1, (_Float16)1, (_Float16)1, (_Float16)1, (_Float16)1, (_Float16)1, (_Float16)1, (_Float16)1};
-          v16f dacc;
+          // row sums of the ROUNDED P (the reference sums them on the tensor cores, rowsum_f16f16f32, attn_utils.cuh:614):
+          // v_dot2_f32_f16 with a pair of ones adds two fp16 values to a binary32 accumulator per instruction, which
+          // leaves the matrix unit to the two products.  Each half-lane sums its own 32 keys; the halves meet in the
+          // epilogue.
+          const h2 ones2 = {(_Float16)1, (_Float16)1};
+          float rs = 0.f;
 #pragma unroll
-          for (int e = 0; e < 16; e++) dacc[e] = 0.f;
+          for (int s4 = 0; s4 < 4; s4++)
 #pragma unroll
-          for (int s4 = 0; s4 < 4; s4++) dacc = __builtin_amdgcn_mfma_f32_32x32x16_f16(ones, pb16[s4], dacc, 0, 0, 0);
-          dsum += dacc[0];                 // all 64 keys of the block, identical in both half-lanes of the query
+            for (int j = 0; j < 8; j += 2) {
+              const h2 pr = {pb16[s4][j], pb16[s4][j + 1]};
+              rs = __builtin_amdgcn_fdot2(pr, ones2, rs, false);
+            }
+          dsum += rs;
         }
+        // V^T operands in two halves of two 16-key steps each, through ONE set of registers (the budget of three
+        // wavefronts per SIMD); every read carries its wait
         const uint32_t va = lds_v0 + 2 * bufoff + v_rd16;
-        v4i t[4][NDT];
-        // steps 0,1 are read first; steps 2,3 are in flight while 0,1 multiply
-        if constexpr (NDT == 4)
-          lds_read_8x128_wait<0, 4096, 8192, 12288>(t[0][0], t[0][1], t[0][2], t[0][3], t[1][0], t[1][1], t[1][2], t[1][3], va, va ^ 16u);
-        else
-          lds_read_4x128_wait<0, 4096>(t[0][0], t[0][1], t[1][0], t[1][1], va, va ^ 16u);
 #pragma unroll
-        for (int s4 = 2; s4 < 4; s4++) {
-          lds_read_2x128<0, 4096>(t[s4][0], t[s4][1], va ^ (uint32_t)(16 * s4));
-          if constexpr (NDT == 4) lds_read_2x128<8192, 12288>(t[s4][2], t[s4][3], va ^ (uint32_t)(16 * s4));
+        for (int half = 0; half < 2; half++) {
+          v4i t[2][NDT];
+          const uint32_t va0 = va ^ (uint32_t)(32 * half), va1 = va0 ^ 16u;
+          if constexpr (NDT == 4)
+            lds_read_8x128_wait<0, 4096, 8192, 12288>(t[0][0], t[0][1], t[0][2], t[0][3], t[1][0], t[1][1], t[1][2], t[1][3], va0, va1);
+          else
+            lds_read_4x128_wait<0, 4096>(t[0][0], t[0][1], t[1][0], t[1][1], va0, va1);
+#pragma unroll
+          for (int u = 0; u < 2; u++)
+#pragma unroll
+            for (int dt = 0; dt < NDT; dt++)
+              O[dt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(h8, t[u][dt]), pb16[2 * half + u], O[dt], 0, 0, 0);
         }
-#pragma unroll
-        for (int s4 = 0; s4 < 2; s4++)
-#pragma unroll
-          for (int dt = 0; dt < NDT; dt++)
-            O[dt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(h8, t[s4][dt]), pb16[s4], O[dt], 0, 0, 0);
-        if constexpr (NDT == 4) { lds_wait4(t[2][0], t[2][1], t[2][2], t[2][3]); lds_wait4(t[3][0], t[3][1], t[3][2], t[3][3]); }
-        else { lds_wait4(t[2][0], t[2][1], t[3][0], t[3][1]); }
-#pragma unroll
-        for (int s4 = 2; s4 < 4; s4++)
-#pragma unroll
-          for (int dt = 0; dt < NDT; dt++)
-            O[dt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(h8, t[s4][dt]), pb16[s4], O[dt], 0, 0, 0);
       } else {
       dsum += ps;
       v8i pb;
@@ -572,7 +603,7 @@ __global__ __launch_bounds__(256, PV16 ? 2 : 3) void block_sparse_attn_kernel(co
     // advance the block pipeline and the ring
     blk = blk1; blk1 = blk2; blk2 = blk2 + d3; d3 = d4;
     ksc = ksc1; ksc1 = ksc2;
-    if constexpr (!CS) bufoff = bufoff == 2 * TILE ? 0 : bufoff + TILE;
+    if constexpr (!CS) bufoff = bufoff == (NBUF - 1) * TILE ? 0 : bufoff + TILE;
   };
   {
     int it = 0;
@@ -590,6 +621,10 @@ __global__ __launch_bounds__(256, PV16 ? 2 : 3) void block_sparse_attn_kernel(co
     for (; it < nv; it++) step(std::true_type{}, std::integral_constant<int, -1>{}, it);
   }
 #undef SPG_LOAD_TILES
+#undef SPG_LOAD_K
+#undef SPG_LOAD_V
+#undef SPG_LOAD_K_
+#undef SPG_LOAD_V_
 #undef SPG_LANE_OFFSETS
 
   // one count per wavefront of 32 query rows, the layout of the reference's PV_Count (sm89.cuh:650-659); the four
@@ -597,7 +632,7 @@ __global__ __launch_bounds__(256, PV16 ? 2 : 3) void block_sparse_attn_kernel(co
   if (p.pv_count != nullptr && lane == 0) p.pv_count[((size_t)bh * p.nq + qb) * 4 + wave] = cnt;
 
   // ---- epilogue: O / d * v_scale -> out dtype -----------------------------------------------------------
-  const float dtot = PV16 ? dsum : half_swap_sum_f32(dsum);
+  const float dtot = half_swap_sum_f32(dsum);
   const float inv = __builtin_amdgcn_rcpf(dtot);
   if (q_row < N) {
     uint16_t *orow = (uint16_t *)p.out + (size_t)(bh / p.H) * p.os.sb + (size_t)head * p.os.sh + (size_t)q_row * p.os.sn;
