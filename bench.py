@@ -25,9 +25,28 @@ PEAK_MFMA_8BIT = 5.0e15   # MI355X dense INT8 = FP8 MFMA peak, op/s
 PEAK_MFMA_F16 = 2.5e15    # MI355X dense FP16 MFMA peak, flop/s
 PEAK_HBM = 8.0e12
 # HBM-side bytes per launch of the attention kernel, measured with two rocprofv3 --pmc runs (FETCH_SIZE, WRITE_SIZE,
-# each scaled by what the same counter reads for a 1 GiB device copy: x2.0 and x1.0).  Only known for the workload
-# it was measured on.
-MEASURED_ATTN_TRAFFIC = {"cfg4": int((1.877 + 0.250) * 2 ** 30)}
+# each scaled by what the same counter reads for a 1 GiB device copy: x2.0 and x1.0).  Only known for the workload it
+# was measured on AND for the kernel source it was measured with: the entry carries the SHA-256 of csrc/attn.hip at
+# the time of the measurement, and the bench line reports the figure only while the source still has that digest.
+MEASURED_ATTN_TRAFFIC = {
+    "cfg4": {"bytes": int((1.894 + 0.250) * 2 ** 30), "attn_hip_sha256": "9d3835bafde519dec8ed5b1f64fe12aa40221642b738c159112c255c267f55b1",
+             "profile": "profiles/cfg4_attn_kernel_pmc.md"},
+}
+
+
+def measured_traffic(cfg_name):
+    """(bytes or None, note) for the roofline's traffic field."""
+    import hashlib
+    ent = MEASURED_ATTN_TRAFFIC.get(cfg_name)
+    if ent is None:
+        return None, "not measured for this workload"
+    src = os.path.join(ROOT, "spargeattn_amd", "csrc", "attn.hip")
+    digest = hashlib.sha256(open(src, "rb").read()).hexdigest()
+    if digest != ent["attn_hip_sha256"]:
+        return None, (f"{ent['profile']} was measured with another version of csrc/attn.hip (sha256 "
+                      f"{ent['attn_hip_sha256'][:12]}, now {digest[:12]}): re-measure")
+    return ent["bytes"], (f"constant: rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of this kernel on this workload, scaled by a "
+                          f"1 GiB copy ({ent['profile']}, csrc/attn.hip sha256 {digest[:12]}); not measured by this run")
 
 
 def parse():
@@ -227,9 +246,8 @@ def main():
                      "bound": "mfma",
                      "achieved": executed_ops / attn_s / 1e12, "peak": peak_mfma / 1e12, "unit": "TFLOP/s",
                      "frac": executed_ops / attn_s / peak_mfma,
-                     "traffic": None if sage1 else MEASURED_ATTN_TRAFFIC.get(cfg.name),
-                     "traffic_source": "constant: rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of this kernel on this workload, "
-                                       "scaled by a 1 GiB copy (profiles/cfg4_attn_kernel_pmc.md); not measured by this run",
+                     "traffic": None if sage1 else measured_traffic(cfg.name)[0],
+                     "traffic_source": "fp16-PV variant: not measured" if sage1 else measured_traffic(cfg.name)[1],
                      "note": "achieved = executed MFMA ops of both products (selected blocks * 2*128*64*D*2) / mean HIP-event "
                              "time of the kernel over the timed steps; peak = MI355X dense 8-bit MFMA"
                              + (" for QK^T and dense fp16 MFMA for PV, blended" if sage1 else "")},
@@ -238,10 +256,18 @@ def main():
     # ---- accuracy of the operator output on sampled Q blocks: against dense fp32 attention on the original tensors
     #      (includes the effect of dropping blocks) and against fp32 attention restricted to the selected blocks -------
     o = step()
+    o_pw = op(q, k, v, is_causal=cfg.is_causal, topk=cfg.topk, pvthreshd=cfg.pvthreshd, qk_quant_gran=2)
+    # per-warp granularity of Q (one INT8 scale per 32 query rows): same kernels, same time - measured here on a few steps
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(max(3, args.steps // 2)):
+        op(q, k, v, is_causal=cfg.is_causal, topk=cfg.topk, pvthreshd=cfg.pvthreshd, qk_quant_gran=2)
+    torch.cuda.synchronize()
+    pw_ms = (time.perf_counter() - t0) / max(3, args.steps // 2) * 1e3
     km = _lib.km_mean(k)
     lut, valid, *_ = utils.get_block_map_meansim_fuse_quant(q, k, km, is_causal=cfg.is_causal, simthreshd1=-0.1,
                                                             cdfthreshd=None, topk=cfg.topk, return_lut=True)
-    num = {"dense": [0.0, 0.0, 0.0, 0.0, 0.0], "masked": [0.0, 0.0, 0.0, 0.0, 0.0]}
+    num = {"dense": [0.0, 0.0, 0.0, 0.0, 0.0], "masked": [0.0, 0.0, 0.0, 0.0, 0.0], "masked_pw": [0.0, 0.0, 0.0, 0.0, 0.0]}
     samples = [(0, nq // 2), (H // 2, nq - 1), (H - 1, nq // 5)]
     for (h, qb) in samples:
         r0, r1 = qb * 128, min(N, qb * 128 + 128)
@@ -253,8 +279,9 @@ def main():
         bm = torch.zeros(nk, dtype=torch.bool, device=dev)
         bm[idx] = True
         tok = bm.repeat_interleave(64)[:N]
-        got = o[0, h, r0:r1].float()
-        for name, scores in (("dense", sc), ("masked", sc.masked_fill(~tok[None, :], float("-inf")))):
+        sc_m = sc.masked_fill(~tok[None, :], float("-inf"))
+        for name, scores, got in (("dense", sc, o[0, h, r0:r1].float()), ("masked", sc_m, o[0, h, r0:r1].float()),
+                                  ("masked_pw", sc_m, o_pw[0, h, r0:r1].float())):
             ref = torch.softmax(scores, dim=-1) @ v[0, h].float()
             a = num[name]
             a[0] += float((got * ref).sum()); a[1] += float((got * got).sum()); a[2] += float((ref * ref).sum())
@@ -268,8 +295,14 @@ def main():
         "vs_fp32_attention_on_selected_blocks": {"cos": num["masked"][0] / (num["masked"][1] * num["masked"][2]) ** 0.5,
                                                  "rel_l1": num["masked"][3] / num["masked"][4]},
         "vs_dense_fp32_sdpa": {"cos": num["dense"][0] / (num["dense"][1] * num["dense"][2]) ** 0.5,
-                               "rel_l1": num["dense"][3] / num["dense"][4]}}
-    del o, lut, valid, km
+                               "rel_l1": num["dense"][3] / num["dense"][4]},
+        "per_warp_q_scales": {"note": "qk_quant_gran=2 (opt-in keyword; the default above is the reference's per-block granularity): "
+                                      "same block map, Q quantised with one scale per 32 rows",
+                              "ms_per_step": pw_ms,
+                              "vs_fp32_attention_on_selected_blocks": {
+                                  "cos": num["masked_pw"][0] / (num["masked_pw"][1] * num["masked_pw"][2]) ** 0.5,
+                                  "rel_l1": num["masked_pw"][3] / num["masked_pw"][4]}}}
+    del o, o_pw, lut, valid, km
 
     if not args.no_dense:
         qh, kh, vh = q.to(torch.float16), k.to(torch.float16), v.to(torch.float16)

@@ -18,7 +18,10 @@
 //  * V lives in HBM as [nk][D][64] e4m3 tiles (one contiguous 64*D-byte read per block), K as (N,D) int8 rows;
 //  * K/V tiles go HBM/L2 -> LDS directly (global_load_lds_dwordx4, no VGPR staging) through a 3-deep LDS ring:
 //    the tiles of block it+2 are in flight while block it is computed, and ONE workgroup barrier per block covers
-//    both the tile hand-over and the workgroup-wide PV-skip vote;
+//    both the tile hand-over and the workgroup-wide PV-skip vote (the FP16-PV variant, whose V^T tiles are twice as
+//    large, uses two-slot rings so that three workgroups still share a CU);
+//  * the INT8 scale of Q is read per 128-row block or per wavefront of 32 rows (qk_quant_gran 1 / 2): a wavefront IS
+//    the 32-row group, so the scale stays a scalar either way;
 //  * LDS tiles are unpadded; bank conflicts are avoided by an XOR swizzle of the 16-byte chunks inside a row
 //    (applied to the per-lane global address for K, baked into the HBM tile layout for V);
 //  * the INT8 accumulators start at the bit pattern of the float 1/(2 pi), an inline constant of the instruction set (no
