@@ -66,7 +66,7 @@ def test_random_case(case):
 
 def _cases_wide():
     """Second sweep: fewer K/V heads than query heads, a key/value length of its own, input magnitudes from 0.1 to 200
-    and both operators (FP8 PV and FP16 PV)."""
+    both operators (FP8 PV and FP16 PV) and both INT8 granularities of Q."""
     rng = np.random.default_rng(20250913)
     out = []
     for i in range(24):
@@ -94,6 +94,8 @@ def test_random_case_grouped_heads_and_lengths(case):
     v = torch.randn((B, Hkv, Nk, D), generator=g).to(dtype)
     kw = dict(topk=level, cdfthreshd=None) if mode == "topk" else dict(topk=None, cdfthreshd=level)
     sim = -0.1 if mode == "topk" else 0.3
+    gran = 2 if i % 2 else 1                 # every other case with per-warp INT8 scales of Q
+    kw["qk_quant_gran"] = gran
     if sage1:
         res = oapi.spas_sage_attn_meansim_topk(to_np(q), to_np(k), to_np(v), tag_of(dtype), is_causal=causal,
                                                simthreshd1=sim, pvthreshd=pvthr, attention_sink=sink, **kw)
@@ -102,7 +104,8 @@ def test_random_case_grouped_heads_and_lengths(case):
         res = oapi.spas_sage2_attn_meansim_topk(to_np(q), to_np(k), to_np(v), tag_of(dtype), is_causal=causal,
                                                 simthreshd1=sim, pvthreshd=pvthr, attention_sink=sink, **kw)
         op = sa.spas_sage2_attn_meansim_topk_cuda if mode == "topk" else sa.spas_sage2_attn_meansim_cuda
-    args = dict(is_causal=causal, simthreshd1=sim, pvthreshd=pvthr, attention_sink=sink, return_sparsity=True)
+    args = dict(is_causal=causal, simthreshd1=sim, pvthreshd=pvthr, attention_sink=sink, return_sparsity=True,
+                qk_quant_gran=gran)
     args["topk" if mode == "topk" else "cdfthreshd"] = level
     qg, kg, vg = q.cuda(), k.cuda(), v.cuda()
     km = _lib.km_mean(kg)
@@ -111,6 +114,7 @@ def test_random_case_grouped_heads_and_lengths(case):
     assert lut.shape == (B, H, (Nq + 127) // 128, (Nk + 63) // 64)
     assert np.array_equal(lut.cpu().numpy(), res["lut"]) and np.array_equal(valid.cpu().numpy(), res["valid"])
     assert np.array_equal(q8.cpu().numpy(), res["q8"]) and np.array_equal(k8.cpu().numpy(), res["k8"])
+    assert np.array_equal(qs.cpu().numpy(), res["q_scale"]) and np.array_equal(ks.cpu().numpy(), res["k_scale"])
     o, sparsity = op(qg, kg, vg, **args)
     assert o.shape == q.shape and abs(sparsity - res["sparsity"]) < 1e-6
     assert torch.isfinite(o.float()).all()
